@@ -1,0 +1,153 @@
+/* sd3_hip.h -- C ABI of the MI355X (gfx950) implementation of the SD3.5-medium MMDiT-X denoiser forward.
+ *
+ * Every entry point replaces one function of MichelHUANGGit/SD3.c `modules.cpp` (cited per declaration) and
+ * keeps its argument meaning, tensor layouts and in-place behaviour. Differences that hold everywhere:
+ *   - all data pointers are DEVICE pointers (HIP global memory), fp32 unless the name says otherwise;
+ *   - a trailing `void* stream` is the hipStream_t to enqueue on (NULL = the default stream); calls are
+ *     asynchronous with respect to the host;
+ *   - the return value is an sd3_status (0 = ok); the library never calls exit() or abort(). The text of the
+ *     last failure on the calling thread is returned by sd3_last_error().
+ * Linear weights use the reference's layout: (C_in, C_out) row-major, i.e. the transposed PyTorch weight
+ * (module_tests/DiT.py:26-31).
+ */
+#ifndef SD3_HIP_H
+#define SD3_HIP_H
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum sd3_status {
+    SD3_OK = 0,
+    SD3_ERR_INVALID_ARG = 1,   /* null pointer, non-positive size, C %% heads != 0 ... */
+    SD3_ERR_MISSING_PARAM = 2, /* a weight the requested configuration needs was not bound */
+    SD3_ERR_UNSUPPORTED = 3,   /* shape outside what the kernels handle (e.g. head_dim > 128) */
+    SD3_ERR_HIP = 4,           /* a HIP runtime call failed; see sd3_last_error() */
+    SD3_ERR_OOM = 5
+} sd3_status;
+
+typedef enum sd3_precision {
+    SD3_PREC_F32 = 0, /* fp32 storage and fp32 MFMA arithmetic: matches the CPU reference to <= 1e-4 */
+    SD3_PREC_BF16 = 1 /* bf16 operands on the MFMA units, fp32 accumulation, fp32 residual stream */
+} sd3_precision;
+
+typedef enum sd3_activation { SD3_ACT_SILU = 0, SD3_ACT_GELU_TANH = 1 } sd3_activation;
+
+typedef struct sd3_ctx sd3_ctx; /* owns: bound weights table, bf16 weight copies, workspace, stream */
+
+const char* sd3_last_error(void);
+int sd3_version(void);
+
+/* ------------------------------------------------------------------ primitive operators (modules.cpp L1) */
+
+/* modules.cpp:10 layernorm(x,y,mean,rstd,w,bias,eps,B,T,C). mean/rstd/w/bias may each be NULL, as in the reference. */
+int sd3_layernorm(const float* x, float* y, float* mean, float* rstd, const float* w, const float* bias, float eps, int B, int T, int C, void* stream);
+/* modules.cpp:154 rmsnorm(x,y,w,rms,eps,B,T,C); x == y allowed. */
+int sd3_rmsnorm(const float* x, float* y, const float* w, float* rms, float eps, int B, int T, int C, void* stream);
+/* modules.cpp:192 rmsnorm_group: per-(token, group) RMSNorm over C/groups values with a shared weight of C/groups values. */
+int sd3_rmsnorm_group(const float* x, float* y, const float* w, float* rms, float eps, int groups, int B, int T, int C, void* stream);
+/* modules.cpp:293 gelu_tanh(input, output, n). */
+int sd3_gelu_tanh(const float* in, float* out, long long n, void* stream);
+/* modules.cpp:352 silu(x, y, n). */
+int sd3_silu(const float* in, float* out, long long n, void* stream);
+/* modules.cpp:475 linear(x,W,b,y,B,C_in,C_out): y = x @ W + b. */
+int sd3_linear(const float* x, const float* W, const float* b, float* y, int B, int C_in, int C_out, void* stream);
+/* modules.cpp:492 partial_linear(x,W,b,y,M,K,N,Nmax,n0): y = x @ W[:, n0:n0+N] + b[n0:n0+N]. */
+int sd3_partial_linear(const float* x, const float* W, const float* b, float* y, int M, int K, int N, int Nmax, int n0, void* stream);
+/* modules.cpp:513 add(input, other, output, size). */
+int sd3_add(const float* a, const float* b, float* out, long long n, void* stream);
+/* modules.cpp:766 multihead_attention(Q,K,V,output,B,num_heads,T,L,head_dim); layouts (B,T,C)/(B,L,C), head h at
+ * columns [h*head_dim,(h+1)*head_dim); output may alias Q. head_dim <= 128. */
+int sd3_multihead_attention(const float* Q, const float* K, const float* V, float* out, int B, int num_heads, int T, int L, int head_dim, void* stream);
+/* modules.cpp:920 sinusoidal_embedding(timesteps, emb_dim): out (B, emb_dim) = [cos | sin]. */
+int sd3_sinusoidal_embedding(const float* timesteps, float* out, int B, int emb_dim, void* stream);
+/* modules.cpp:946 positional_embedding2D(output, emb_dim, height, width, base_size); table evaluated in fp64. */
+int sd3_positional_embedding2D(float* out, int emb_dim, int height, int width, int base_size, void* stream);
+/* modules.cpp:977 crop_positional_embedding2D(pos_embed, new_pos_embed, pos_embed_max_size, new_height, new_width, emb_dim). */
+int sd3_crop_positional_embedding2D(const float* pos_embed, float* out, int pos_embed_max_size, int new_height, int new_width, int emb_dim, void* stream);
+/* modules.cpp:1037 conv2d(...). Unlike the reference, `output` need not be zeroed by the caller. */
+int sd3_conv2d(const float* in, float* out, const float* kernel, const float* bias, int B, int kernel_height, int kernel_width, int in_channels,
+               int out_channels, int in_height, int in_width, int out_height, int out_width, int stride, int padding, void* stream);
+/* modules.cpp:1093 PatchEmbedding(latent, patches, pos_embed_max, pos_embed, output, kernel, bias, B,H,W,C,emb_dim,patch,pos_max,base_height).
+ * The three scratch pointers of the reference are not needed: the kernel gathers patches itself and the
+ * position table of the requested grid is generated on the device. */
+int sd3_patch_embedding(const float* latent, float* out, const float* kernel, const float* bias, int B, int H, int W, int C_in, int emb_dim,
+                        int patch_size, int pos_embed_max_size, int base_height, void* stream);
+/* modules.cpp:1120 mlp(x, output, h1, W1,b1,W2,b2, B,C_in,C_hid,C_out, activation); the std::function becomes an sd3_activation. */
+int sd3_mlp(const float* x, float* out, float* h1, const float* W1, const float* b1, const float* W2, const float* b2, int B, int C_in, int C_hid,
+            int C_out, int activation, void* stream);
+/* modules.cpp:1207 scale_and_shift(input, output, shift, scale, B,T,C): out = in*(1+scale[b]) + shift[b]. */
+int sd3_scale_and_shift(const float* in, float* out, const float* shift, const float* scale, int B, int T, int C, void* stream);
+/* modules.cpp:1223 gating_mechanism(input, output, gate, B,T,C). */
+int sd3_gating_mechanism(const float* in, float* out, const float* gate, int B, int T, int C, void* stream);
+/* modules.cpp:1239 / 1268 concatenate_along_tokens / split_along_tokens. */
+int sd3_concatenate_along_tokens(const float* x, const float* y, float* out, int B, int Tx, int Ty, int C, void* stream);
+int sd3_split_along_tokens(const float* in, float* split1, float* split2, int B, int T1, int T2, int C, void* stream);
+
+/* ------------------------------------------------------------------ the block with raw pointers (modules.cpp L2) */
+
+/* Weights of one block in the argument order of dit_block (modules.cpp:1344-1358). Absent entries are NULL and are
+ * never dereferenced (last block: no context out-projection / MLP; non-dual blocks: no x2_*; no qk-norm: no *_rms_*). */
+typedef struct sd3_block_weights {
+    const float *c_ada_w, *c_ada_b, *c_qkv_w, *c_qkv_b, *c_rms_q, *c_rms_k, *c_out_w, *c_out_b, *c_mlp_w1, *c_mlp_b1, *c_mlp_w2, *c_mlp_b2;
+    const float *x_ada_w, *x_ada_b, *x_qkv_w, *x_qkv_b, *x_rms_q, *x_rms_k, *x_out_w, *x_out_b;
+    const float *x2_qkv_w, *x2_qkv_b, *x2_rms_q, *x2_rms_k, *x2_out_w, *x2_out_b;
+    const float *x_mlp_w1, *x_mlp_b1, *x_mlp_w2, *x_mlp_b2;
+} sd3_block_weights;
+
+/* modules.cpp:1340 dit_block(y, c, x, <30 weights>, <16 scratch>, B,Tc,Tx,emb_dim,attn_heads,mlp_expand,use_dual,use_qk_norm,discard).
+ * c and x are updated in place. The reference's 16 caller-owned scratch buffers are replaced by the context's
+ * workspace (the fused kernels use differently shaped intermediates). */
+int sd3_dit_block_w(sd3_ctx* ctx, const float* y, float* c, float* x, const sd3_block_weights* w, int B, int Tc, int Tx, int emb_dim,
+                    int attn_heads, int mlp_expand, int use_dual_attention, int use_qk_norm, int discard_context, int precision);
+
+/* ------------------------------------------------------------------ context, weights by name (modules.cpp L3) */
+
+int sd3_ctx_create(sd3_ctx** out, int device);
+int sd3_ctx_destroy(sd3_ctx* ctx);
+int sd3_ctx_set_stream(sd3_ctx* ctx, void* stream);
+int sd3_ctx_synchronize(sd3_ctx* ctx);
+
+/* One entry of the reference's `name -> tensor` parameter map (modules.cpp:1512,1609). `ptr` is borrowed: it must stay
+ * valid and unchanged while bound. Names are the reference's (modules.cpp:1558-1575, 1665-1728). */
+int sd3_weights_bind(sd3_ctx* ctx, const char* name, const float* ptr, long long numel);
+int sd3_weights_clear(sd3_ctx* ctx);
+/* Builds (or refreshes) the bf16 MFMA copies of every bound 2-D weight ahead of time. Optional: they are otherwise
+ * built on first use. `emb_dim` etc. tell the library which bound tensors are GEMM weights and their shapes. */
+int sd3_weights_prepare(sd3_ctx* ctx, int precision);
+
+/* modules.cpp:1508 DiT_block_forward / modules.cpp:1783 DiT_block_forward_cuda: the block with weights looked up by
+ * name. `prefix` is "" for the single-block entry points and "transformer.<l>." inside the full model. */
+int sd3_dit_block(sd3_ctx* ctx, const float* y, float* c, float* x, const char* prefix, int B, int Tc, int Tx, int emb_dim, int attn_heads,
+                  int mlp_expand, int use_dual_attention, int use_qk_norm, int discard_context, int precision);
+
+/* modules.cpp:1605 DiT_forward(pooled_captions, captions, latent_vector, timesteps, params, num_layers, dual_attention_layers,
+ * pooled_dim, captions_dim, C_in, emb_dim, attn_heads, mlp_expand, patch_size, pos_embed_max_size, base_height, use_qk_norm).
+ * pooled (B,pooled_dim), captions (B,Tc,captions_dim), latent (B,C_in,H,W), timesteps (B); out (B,C_in,H,W). Inputs are
+ * left untouched. The std::unordered_set of dual layers becomes an int array. */
+int sd3_dit_forward(sd3_ctx* ctx, const float* pooled, const float* captions, const float* latent, const float* timesteps, float* out, int B,
+                    int Tc, int H, int W, int num_layers, const int* dual_attention_layers, int n_dual, int pooled_dim, int captions_dim, int C_in,
+                    int emb_dim, int attn_heads, int mlp_expand, int patch_size, int pos_embed_max_size, int base_height, int use_qk_norm,
+                    int precision);
+
+/* ------------------------------------------------------------------ bf16 kernels on their own (no counterpart in the reference,
+ * whose GPU file is fp32/TF32 only; exposed so that the MFMA kernels can be tested and timed in isolation) */
+
+/* Joint attention over two token segments without concatenation: segment 0 (context, T0 tokens) then segment 1
+ * (latent, T1 tokens), each given as a packed bf16 (B*T_s, 3*C) q|k|v buffer as the QKV GEMM writes it. Per-head
+ * RMSNorm (eps 1e-6, weights rms_q[s]/rms_k[s] of head_dim floats, or NULL for none) is applied to q and k while
+ * they are loaded. Output: bf16 (B*T_s, C) per segment (out[s] may be NULL to skip writing it). head_dim must be 64.
+ * This is the fused form of modules.cpp:1396-1399,1420-1432 (rmsnorm_group x4, concatenate x3, attention, split). */
+int sd3_flash_attention_bf16(const void* qkv0, const void* qkv1, void* out0, void* out1, const float* rms_q0, const float* rms_k0,
+                             const float* rms_q1, const float* rms_k1, int B, int T0, int T1, int num_heads, int head_dim, void* stream);
+/* out(M,N) = A(M,K) @ W + bias with A bf16 row-major, W given in the reference's fp32 (K,N) layout already packed by
+ * sd3_pack_weight_bf16 into `wpacked`; out bf16. K %% 64 == 0 and N %% 8 == 0 required. epilogue: 0 bias, 1 bias+GELU-tanh. */
+int sd3_pack_weight_bf16(const float* W, void* wpacked, int K, int N, void* stream);
+int sd3_gemm_bf16(const void* A, const void* wpacked, const float* bias, void* out, int M, int N, int K, int epilogue, void* stream);
+/* fp32 -> bf16 (round to nearest even) */
+int sd3_cast_f32_to_bf16(const float* in, void* out, long long n, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SD3_HIP_H */

@@ -1,0 +1,789 @@
+// Host side of the library: context (bound weights, bf16 copies, workspace), the block schedule
+// (dit_block, modules.cpp:1340-1505) and the full forward (DiT_forward, modules.cpp:1605-1780) expressed as
+// launches of the fused kernels. No arithmetic happens on the host.
+#include <cmath>
+#include <cstring>
+#include <map>
+#include <new>
+#include <string>
+#include <tuple>
+#include <unordered_map>
+#include <vector>
+
+#include "common.hpp"
+
+namespace sd3 {
+
+// ------------------------------------------------------------------ errors
+static thread_local char g_err[512] = "";
+void set_error(const char* msg) {
+    std::strncpy(g_err, msg, sizeof(g_err) - 1);
+    g_err[sizeof(g_err) - 1] = 0;
+}
+int fail(int status, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    std::vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return status;
+}
+const char* last_error() { return g_err; }
+
+}  // namespace sd3
+
+using namespace sd3;
+
+// ------------------------------------------------------------------ context
+struct PackedWeight {
+    void* ptr = nullptr;
+    long long K = 0, N = 0;
+    int kind = 0;  // 0: bf16 (N,K) transposed for the MFMA GEMM; 1: bf16 (K,N) plain cast for small_linear; 2: fp32 (K,N) transpose of an (N,K) tensor
+};
+
+struct sd3_ctx {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    std::unordered_map<std::string, std::pair<const float*, long long>> params;
+    std::map<std::pair<const float*, int>, PackedWeight> packed;
+    std::map<std::tuple<int, int, int, int, int>, float*> pos_tables;  // (C, max, base, h, w) -> cropped table
+    void* ws = nullptr;
+    size_t ws_bytes = 0;
+};
+
+namespace {
+
+struct Bump {
+    char* base;
+    size_t off = 0, cap;
+    Bump(void* b, size_t c) : base((char*)b), cap(c) {}
+    template <typename T>
+    T* take(size_t n) {
+        size_t bytes = (n * sizeof(T) + 255) & ~(size_t)255;
+        T* p = base ? reinterpret_cast<T*>(base + off) : nullptr;
+        off += bytes;
+        return p;
+    }
+};
+
+int ensure_workspace(sd3_ctx* ctx, size_t bytes) {
+    if (bytes <= ctx->ws_bytes) return SD3_OK;
+    if (ctx->ws) {
+        SD3_HIP_TRY(hipStreamSynchronize(ctx->stream));
+        SD3_HIP_TRY(hipFree(ctx->ws));
+        ctx->ws = nullptr;
+        ctx->ws_bytes = 0;
+    }
+    hipError_t e = hipMalloc(&ctx->ws, bytes);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        return fail(SD3_ERR_OOM, "workspace of %zu bytes: %s", bytes, hipGetErrorString(e));
+    }
+    ctx->ws_bytes = bytes;
+    return SD3_OK;
+}
+
+int get_packed(sd3_ctx* ctx, const float* w, long long K, long long N, int kind, const void** out) {
+    auto key = std::make_pair(w, kind);
+    auto it = ctx->packed.find(key);
+    if (it != ctx->packed.end() && it->second.K == K && it->second.N == N) {
+        *out = it->second.ptr;
+        return SD3_OK;
+    }
+    if (it != ctx->packed.end()) {
+        SD3_HIP_TRY(hipStreamSynchronize(ctx->stream));
+        SD3_HIP_TRY(hipFree(it->second.ptr));
+        ctx->packed.erase(it);
+    }
+    PackedWeight p;
+    p.K = K; p.N = N; p.kind = kind;
+    const size_t bytes = (size_t)K * N * (kind == 2 ? 4 : 2);
+    hipError_t e = hipMalloc(&p.ptr, bytes);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        return fail(SD3_ERR_OOM, "bf16 weight copy of %zu bytes: %s", bytes, hipGetErrorString(e));
+    }
+    int rc;
+    if (kind == 0) rc = pack_weight_bf16(w, (bf16_t*)p.ptr, (int)K, (int)N, ctx->stream);
+    else if (kind == 1) rc = cast_f32_to_bf16(w, (bf16_t*)p.ptr, K * N, ctx->stream);
+    else rc = transpose_f32(w, (float*)p.ptr, (int)N, (int)K, ctx->stream);  // input is (N,K): transpose to (K,N)
+    if (rc != SD3_OK) {
+        (void)hipFree(p.ptr);
+        return rc;
+    }
+    ctx->packed[key] = p;
+    *out = p.ptr;
+    return SD3_OK;
+}
+
+struct Dims {
+    int B, Tc, Tx, C, NH, HS, E;  // E = mlp_expand
+    bool dual, qk, discard;
+};
+
+size_t block_workspace_bytes(const Dims& d, int prec) {
+    Bump b(nullptr, 0);
+    const size_t es = prec == SD3_PREC_BF16 ? 2 : 4;
+    const size_t mc = (size_t)d.B * d.Tc, mx = (size_t)d.B * d.Tx;
+    auto act = [&](size_t n) { b.take<char>(n * es); };
+    act(mc * d.C); act(mx * d.C); act(mx * d.C);           // c_hid, x_hid, x_hid2
+    act(mc * 3 * d.C); act(mx * 3 * d.C);                  // c_qkv, x_qkv
+    act(mc * d.C); act(mx * d.C);                          // c_att, x_att
+    act(mc * d.E * d.C); act(mx * d.E * d.C);              // c_mlp, x_mlp
+    b.take<float>((size_t)d.B * 6 * d.C); b.take<float>((size_t)d.B * 9 * d.C);  // ada_c, ada_x
+    return b.off;
+}
+
+// One linear layer: out = epilogue(A @ W + b). fp32: W used in place; bf16: the packed copy.
+int linear_layer(sd3_ctx* ctx, int prec, const void* A, const float* W, const float* bias, void* out, int out_f32, int ldc, int M, int N, int K, int epi,
+                 GemmEpilogueArgs ea) {
+    if (!W) return fail(SD3_ERR_MISSING_PARAM, "a weight needed by this configuration is not bound (N=%d K=%d)", N, K);
+    ea.bias = bias;
+    if (prec == SD3_PREC_F32) return gemm_f32((const float*)A, K, W, N, 0, (float*)out, ldc, M, N, K, epi, ea, ctx->stream);
+    const void* wp = nullptr;
+    SD3_TRY(get_packed(ctx, W, K, N, 0, &wp));
+    return gemm_bf16((const bf16_t*)A, (const bf16_t*)wp, out, out_f32, ldc, M, N, K, epi, ea, ctx->stream);
+}
+
+int ada_jobs_run(sd3_ctx* ctx, int prec, const float* y, int B, int C, std::vector<SmallLinearJob>& jobs) {
+    if (prec == SD3_PREC_BF16) {
+        for (auto& j : jobs) {
+            const void* wp = nullptr;
+            SD3_TRY(get_packed(ctx, (const float*)j.W, C, j.ldw, 1, &wp));
+            j.W = wp;
+        }
+    }
+    return small_linear_batched(y, B, C, jobs.data(), (int)jobs.size(), prec == SD3_PREC_BF16, -1, ctx->stream);
+}
+
+// The block. ada_c / ada_x: modulation vectors (B, chunks*C) already computed, or null to compute them here.
+int run_block(sd3_ctx* ctx, int prec, const float* y, float* c, float* x, const sd3_block_weights& w, const Dims& d, const float* ada_c,
+              const float* ada_x, Bump& ws) {
+    hipStream_t st = ctx->stream;
+    const int B = d.B, Tc = d.Tc, Tx = d.Tx, C = d.C;
+    const int mc = B * Tc, mx = B * Tx;
+    const int cch = d.discard ? 2 : 6, xch = d.dual ? 9 : 6;
+    const bool bf = prec == SD3_PREC_BF16;
+    const size_t es = bf ? 2 : 4;
+    auto act = [&](size_t n) -> void* { return ws.take<char>(n * es); };
+    void* c_hid = act((size_t)mc * C);
+    void* x_hid = act((size_t)mx * C);
+    void* x_hid2 = act((size_t)mx * C);
+    void* c_qkv = act((size_t)mc * 3 * C);
+    void* x_qkv = act((size_t)mx * 3 * C);
+    void* c_att = act((size_t)mc * C);
+    void* x_att = act((size_t)mx * C);
+    void* c_mlp = act((size_t)mc * d.E * C);
+    void* x_mlp = act((size_t)mx * d.E * C);
+    float* ada_c_buf = ws.take<float>((size_t)B * 6 * C);
+    float* ada_x_buf = ws.take<float>((size_t)B * 9 * C);
+
+    if (!w.c_ada_w || !w.c_ada_b || !w.x_ada_w || !w.x_ada_b) return fail(SD3_ERR_MISSING_PARAM, "adaLN modulation weights are not bound");
+    if (!w.c_qkv_w || !w.c_qkv_b || !w.x_qkv_w || !w.x_qkv_b || !w.x_out_w || !w.x_out_b || !w.x_mlp_w1 || !w.x_mlp_b1 || !w.x_mlp_w2 || !w.x_mlp_b2)
+        return fail(SD3_ERR_MISSING_PARAM, "attention / MLP weights of the latent or context stream are not bound");
+    if (!d.discard && (!w.c_out_w || !w.c_out_b || !w.c_mlp_w1 || !w.c_mlp_b1 || !w.c_mlp_w2 || !w.c_mlp_b2))
+        return fail(SD3_ERR_MISSING_PARAM, "context out-projection / MLP weights are not bound (needed unless discard_context)");
+    if (d.dual && (!w.x2_qkv_w || !w.x2_qkv_b || !w.x2_out_w || !w.x2_out_b))
+        return fail(SD3_ERR_MISSING_PARAM, "latent_dual_* weights are not bound (needed with use_dual_attention)");
+    if (d.qk && (!w.c_rms_q || !w.c_rms_k || !w.x_rms_q || !w.x_rms_k || (d.dual && (!w.x2_rms_q || !w.x2_rms_k))))
+        return fail(SD3_ERR_MISSING_PARAM, "rmsnorm weights are not bound (needed with use_qk_norm)");
+
+    // modulation vectors: every chunk of both streams in one launch (the reference issues 12-20 partial_linear calls)
+    if (!ada_c || !ada_x) {
+        std::vector<SmallLinearJob> jobs = {
+            {w.c_ada_w, w.c_ada_b, ada_c_buf, cch * C, cch * C, 0},
+            {w.x_ada_w, w.x_ada_b, ada_x_buf, xch * C, xch * C, 0},
+        };
+        SD3_TRY(ada_jobs_run(ctx, prec, y, B, C, jobs));
+        ada_c = ada_c_buf;
+        ada_x = ada_x_buf;
+    }
+    const int ldc_ada = cch * C, ldx_ada = xch * C;
+    auto cchunk = [&](int k) { return ada_c + (size_t)k * C; };
+    auto xchunk = [&](int k) { return ada_x + (size_t)k * C; };
+    GemmEpilogueArgs none;
+
+    // ---- context stream up to q,k,v (modules.cpp:1381-1399); with discard_context chunk 0 is the scale, chunk 1 the shift
+    const float* c_shift = d.discard ? cchunk(1) : cchunk(0);
+    const float* c_scale = d.discard ? cchunk(0) : cchunk(1);
+    SD3_TRY(layernorm_modulate(c, c_hid, nullptr, c_shift, c_scale, nullptr, nullptr, ldc_ada, 1e-6f, B, Tc, C, bf, st));
+    SD3_TRY(linear_layer(ctx, prec, c_hid, w.c_qkv_w, w.c_qkv_b, c_qkv, !bf, 3 * C, mc, 3 * C, C, EPI_BIAS, none));
+    // ---- latent stream up to q,k,v (modules.cpp:1402-1423); the dual branch's input comes from the same normalised rows
+    SD3_TRY(layernorm_modulate(x, x_hid, d.dual ? x_hid2 : nullptr, xchunk(0), xchunk(1), d.dual ? xchunk(6) : nullptr, d.dual ? xchunk(7) : nullptr,
+                               ldx_ada, 1e-6f, B, Tx, C, bf, st));
+    SD3_TRY(linear_layer(ctx, prec, x_hid, w.x_qkv_w, w.x_qkv_b, x_qkv, !bf, 3 * C, mx, 3 * C, C, EPI_BIAS, none));
+
+    // ---- joint attention over [context ; latent] (modules.cpp:1427-1432), qk-norm fused (bf16) or done in place first (fp32)
+    auto seg_ptr = [&](void* base, int third) -> void* { return (char*)base + (size_t)third * C * es; };
+    if (!bf && d.qk) {
+        SD3_TRY(rmsnorm_rows((float*)c_qkv, (float*)c_qkv, w.c_rms_q, nullptr, 1e-6f, mc, d.NH, d.HS, 3 * C, 3 * C, st));
+        SD3_TRY(rmsnorm_rows((float*)seg_ptr(c_qkv, 1), (float*)seg_ptr(c_qkv, 1), w.c_rms_k, nullptr, 1e-6f, mc, d.NH, d.HS, 3 * C, 3 * C, st));
+        SD3_TRY(rmsnorm_rows((float*)x_qkv, (float*)x_qkv, w.x_rms_q, nullptr, 1e-6f, mx, d.NH, d.HS, 3 * C, 3 * C, st));
+        SD3_TRY(rmsnorm_rows((float*)seg_ptr(x_qkv, 1), (float*)seg_ptr(x_qkv, 1), w.x_rms_k, nullptr, 1e-6f, mx, d.NH, d.HS, 3 * C, 3 * C, st));
+    }
+    {
+        AttnSegments a{};
+        a.q[0] = c_qkv; a.k[0] = seg_ptr(c_qkv, 1); a.v[0] = seg_ptr(c_qkv, 2); a.out[0] = d.discard ? nullptr : c_att;
+        a.q[1] = x_qkv; a.k[1] = seg_ptr(x_qkv, 1); a.v[1] = seg_ptr(x_qkv, 2); a.out[1] = x_att;
+        a.ld_qkv[0] = a.ld_qkv[1] = 3 * C; a.ld_out[0] = a.ld_out[1] = C;
+        a.T[0] = a.Tq[0] = Tc; a.T[1] = a.Tq[1] = Tx;
+        if (d.qk) { a.rms_q[0] = w.c_rms_q; a.rms_k[0] = w.c_rms_k; a.rms_q[1] = w.x_rms_q; a.rms_k[1] = w.x_rms_k; }
+        SD3_TRY(bf ? attention_bf16(a, B, d.NH, d.HS, st) : attention_f32(a, B, d.NH, d.HS, st));
+    }
+    // ---- out-projections with the gate and the residual add in the epilogue (modules.cpp:1435-1436, 1459-1462, 1481-1485)
+    GemmEpilogueArgs ge;
+    ge.rows_per_batch = Tc; ge.gate = cchunk(2); ge.gate_ld = ldc_ada; ge.resid = c;
+    if (!d.discard) SD3_TRY(linear_layer(ctx, prec, c_att, w.c_out_w, w.c_out_b, c, 1, C, mc, C, C, EPI_GATE_RESID, ge));
+    ge.rows_per_batch = Tx; ge.gate = xchunk(2); ge.gate_ld = ldx_ada; ge.resid = x;
+    SD3_TRY(linear_layer(ctx, prec, x_att, w.x_out_w, w.x_out_b, x, 1, C, mx, C, C, EPI_GATE_RESID, ge));
+
+    // ---- extra self-attention over the latent tokens (modules.cpp:1440-1453, 1486)
+    if (d.dual) {
+        SD3_TRY(linear_layer(ctx, prec, x_hid2, w.x2_qkv_w, w.x2_qkv_b, x_qkv, !bf, 3 * C, mx, 3 * C, C, EPI_BIAS, none));
+        if (!bf && d.qk) {
+            SD3_TRY(rmsnorm_rows((float*)x_qkv, (float*)x_qkv, w.x2_rms_q, nullptr, 1e-6f, mx, d.NH, d.HS, 3 * C, 3 * C, st));
+            SD3_TRY(rmsnorm_rows((float*)seg_ptr(x_qkv, 1), (float*)seg_ptr(x_qkv, 1), w.x2_rms_k, nullptr, 1e-6f, mx, d.NH, d.HS, 3 * C, 3 * C, st));
+        }
+        AttnSegments a{};
+        a.q[0] = x_qkv; a.k[0] = seg_ptr(x_qkv, 1); a.v[0] = seg_ptr(x_qkv, 2); a.out[0] = x_att;
+        a.ld_qkv[0] = a.ld_qkv[1] = 3 * C; a.ld_out[0] = a.ld_out[1] = C;
+        a.T[0] = a.Tq[0] = Tx;
+        if (d.qk) { a.rms_q[0] = w.x2_rms_q; a.rms_k[0] = w.x2_rms_k; }
+        SD3_TRY(bf ? attention_bf16(a, B, d.NH, d.HS, st) : attention_f32(a, B, d.NH, d.HS, st));
+        ge.rows_per_batch = Tx; ge.gate = xchunk(8); ge.gate_ld = ldx_ada; ge.resid = x;
+        SD3_TRY(linear_layer(ctx, prec, x_att, w.x2_out_w, w.x2_out_b, x, 1, C, mx, C, C, EPI_GATE_RESID, ge));
+    }
+
+    // ---- context MLP (modules.cpp:1463-1476)
+    if (!d.discard) {
+        SD3_TRY(layernorm_modulate(c, c_hid, nullptr, cchunk(3), cchunk(4), nullptr, nullptr, ldc_ada, 1e-6f, B, Tc, C, bf, st));
+        SD3_TRY(linear_layer(ctx, prec, c_hid, w.c_mlp_w1, w.c_mlp_b1, c_mlp, !bf, d.E * C, mc, d.E * C, C, EPI_BIAS_GELU, none));
+        ge.rows_per_batch = Tc; ge.gate = cchunk(5); ge.gate_ld = ldc_ada; ge.resid = c;
+        SD3_TRY(linear_layer(ctx, prec, c_mlp, w.c_mlp_w2, w.c_mlp_b2, c, 1, C, mc, C, d.E * C, EPI_GATE_RESID, ge));
+    }
+    // ---- latent MLP (modules.cpp:1488-1504)
+    SD3_TRY(layernorm_modulate(x, x_hid, nullptr, xchunk(3), xchunk(4), nullptr, nullptr, ldx_ada, 1e-6f, B, Tx, C, bf, st));
+    SD3_TRY(linear_layer(ctx, prec, x_hid, w.x_mlp_w1, w.x_mlp_b1, x_mlp, !bf, d.E * C, mx, d.E * C, C, EPI_BIAS_GELU, none));
+    ge.rows_per_batch = Tx; ge.gate = xchunk(5); ge.gate_ld = ldx_ada; ge.resid = x;
+    SD3_TRY(linear_layer(ctx, prec, x_mlp, w.x_mlp_w2, w.x_mlp_b2, x, 1, C, mx, C, d.E * C, EPI_GATE_RESID, ge));
+    return SD3_OK;
+}
+
+int check_block_dims(const Dims& d, int prec) {
+    if (d.B <= 0 || d.Tc < 0 || d.Tx <= 0 || d.C <= 0 || d.NH <= 0 || d.E <= 0)
+        return fail(SD3_ERR_INVALID_ARG, "block: sizes must be positive (B=%d Tc=%d Tx=%d emb_dim=%d heads=%d mlp_expand=%d)", d.B, d.Tc, d.Tx, d.C, d.NH, d.E);
+    if (d.C % d.NH) return fail(SD3_ERR_INVALID_ARG, "block: emb_dim %d is not divisible by attn_heads %d", d.C, d.NH);
+    if (d.B > 8) return fail(SD3_ERR_UNSUPPORTED, "block: batch %d > 8", d.B);
+    if (prec != SD3_PREC_F32 && prec != SD3_PREC_BF16) return fail(SD3_ERR_INVALID_ARG, "unknown precision %d", prec);
+    if (prec == SD3_PREC_BF16 && (d.HS != 64 || d.C % 64)) return fail(SD3_ERR_UNSUPPORTED, "bf16 path needs head_dim 64 and emb_dim %% 64 == 0");
+    if (prec == SD3_PREC_F32 && d.HS > 128) return fail(SD3_ERR_UNSUPPORTED, "fp32 path needs head_dim <= 128");
+    return SD3_OK;
+}
+
+const float* find_param(sd3_ctx* ctx, const std::string& name, long long expect_numel, int* status) {
+    auto it = ctx->params.find(name);
+    if (it == ctx->params.end()) return nullptr;
+    if (expect_numel > 0 && it->second.second != expect_numel) {
+        *status = fail(SD3_ERR_INVALID_ARG, "parameter %s has %lld elements, expected %lld", name.c_str(), it->second.second, expect_numel);
+        return nullptr;
+    }
+    return it->second.first;
+}
+
+int lookup_block_weights(sd3_ctx* ctx, const std::string& prefix, const Dims& d, sd3_block_weights* w) {
+    int st = SD3_OK;
+    const long long C = d.C, E = d.E;
+    const long long cch = d.discard ? 2 : 6, xch = d.dual ? 9 : 6;
+    auto g = [&](const char* n, long long numel) { return find_param(ctx, prefix + n, numel, &st); };
+    w->c_ada_w = g("context_ada_lnorm.linear.weight", C * cch * C); w->c_ada_b = g("context_ada_lnorm.linear.bias", cch * C);
+    w->c_qkv_w = g("context_to_qkv.weight", C * 3 * C); w->c_qkv_b = g("context_to_qkv.bias", 3 * C);
+    w->c_rms_q = g("context_rmsnorm_query.weight", d.HS); w->c_rms_k = g("context_rmsnorm_key.weight", d.HS);
+    w->c_out_w = g("context_attn_Wout.weight", C * C); w->c_out_b = g("context_attn_Wout.bias", C);
+    w->c_mlp_w1 = g("context_mlp.lin1.weight", C * E * C); w->c_mlp_b1 = g("context_mlp.lin1.bias", E * C);
+    w->c_mlp_w2 = g("context_mlp.lin2.weight", C * E * C); w->c_mlp_b2 = g("context_mlp.lin2.bias", C);
+    w->x_ada_w = g("latent_ada_lnorm.linear.weight", C * xch * C); w->x_ada_b = g("latent_ada_lnorm.linear.bias", xch * C);
+    w->x_qkv_w = g("latent_to_qkv.weight", C * 3 * C); w->x_qkv_b = g("latent_to_qkv.bias", 3 * C);
+    w->x_rms_q = g("latent_rmsnorm_query.weight", d.HS); w->x_rms_k = g("latent_rmsnorm_key.weight", d.HS);
+    w->x_out_w = g("latent_attn_Wout.weight", C * C); w->x_out_b = g("latent_attn_Wout.bias", C);
+    w->x2_qkv_w = g("latent_dual_to_qkv.weight", C * 3 * C); w->x2_qkv_b = g("latent_dual_to_qkv.bias", 3 * C);
+    w->x2_rms_q = g("latent_dual_rmsnorm_query.weight", d.HS); w->x2_rms_k = g("latent_dual_rmsnorm_key.weight", d.HS);
+    w->x2_out_w = g("latent_dual_attn_Wout.weight", C * C); w->x2_out_b = g("latent_dual_attn_Wout.bias", C);
+    w->x_mlp_w1 = g("latent_mlp.lin1.weight", C * E * C); w->x_mlp_b1 = g("latent_mlp.lin1.bias", E * C);
+    w->x_mlp_w2 = g("latent_mlp.lin2.weight", C * E * C); w->x_mlp_b2 = g("latent_mlp.lin2.bias", C);
+    return st;
+}
+
+struct DeviceGuard {
+    int prev = -1;
+    bool ok = false;
+    explicit DeviceGuard(int dev) {
+        if (hipGetDevice(&prev) == hipSuccess && (prev == dev || hipSetDevice(dev) == hipSuccess)) ok = true;
+        else (void)hipGetLastError();
+    }
+    ~DeviceGuard() {
+        int cur = -1;
+        if (ok && hipGetDevice(&cur) == hipSuccess && cur != prev) (void)hipSetDevice(prev);
+    }
+};
+
+}  // namespace
+
+// ================================================================== C ABI
+extern "C" {
+
+const char* sd3_last_error(void) { return sd3::last_error(); }
+int sd3_version(void) { return 1; }
+
+#define ST(s) ((hipStream_t)(s))
+#define NOTNULL(p) SD3_REQUIRE((p) != nullptr, "%s: null pointer argument '%s'", __func__, #p)
+
+int sd3_layernorm(const float* x, float* y, float* mean, float* rstd, const float* w, const float* bias, float eps, int B, int T, int C, void* stream) {
+    SD3_REQUIRE(B >= 0 && T >= 0 && C > 0, "layernorm: bad sizes B=%d T=%d C=%d", B, T, C);
+    if ((long long)B * T == 0) return SD3_OK;
+    NOTNULL(x); NOTNULL(y);
+    return layernorm_full(x, y, mean, rstd, w, bias, eps, (long long)B * T, C, ST(stream));
+}
+int sd3_rmsnorm(const float* x, float* y, const float* w, float* rms, float eps, int B, int T, int C, void* stream) {
+    SD3_REQUIRE(B >= 0 && T >= 0 && C > 0, "rmsnorm: bad sizes B=%d T=%d C=%d", B, T, C);
+    if ((long long)B * T == 0) return SD3_OK;
+    NOTNULL(x); NOTNULL(y);
+    return rmsnorm_rows(x, y, w, rms, eps, (long long)B * T, 1, C, C, C, ST(stream));
+}
+int sd3_rmsnorm_group(const float* x, float* y, const float* w, float* rms, float eps, int groups, int B, int T, int C, void* stream) {
+    SD3_REQUIRE(B >= 0 && T >= 0 && C > 0 && groups > 0, "rmsnorm_group: bad sizes B=%d T=%d C=%d groups=%d", B, T, C, groups);
+    SD3_REQUIRE(C % groups == 0, "rmsnorm_group: C=%d is not divisible by groups=%d", C, groups);
+    if ((long long)B * T == 0) return SD3_OK;
+    NOTNULL(x); NOTNULL(y);
+    return rmsnorm_rows(x, y, w, rms, eps, (long long)B * T, groups, C / groups, C, C, ST(stream));
+}
+int sd3_gelu_tanh(const float* in, float* out, long long n, void* stream) {
+    SD3_REQUIRE(n >= 0, "gelu_tanh: negative size");
+    if (n == 0) return SD3_OK;
+    NOTNULL(in); NOTNULL(out);
+    return unary_op(in, out, n, SD3_ACT_GELU_TANH, ST(stream));
+}
+int sd3_silu(const float* in, float* out, long long n, void* stream) {
+    SD3_REQUIRE(n >= 0, "silu: negative size");
+    if (n == 0) return SD3_OK;
+    NOTNULL(in); NOTNULL(out);
+    return unary_op(in, out, n, SD3_ACT_SILU, ST(stream));
+}
+int sd3_linear(const float* x, const float* W, const float* b, float* y, int B, int C_in, int C_out, void* stream) {
+    SD3_REQUIRE(B >= 0 && C_in > 0 && C_out > 0, "linear: bad sizes B=%d C_in=%d C_out=%d", B, C_in, C_out);
+    if (B == 0) return SD3_OK;
+    NOTNULL(x); NOTNULL(W); NOTNULL(b); NOTNULL(y);
+    GemmEpilogueArgs ea;
+    ea.bias = b;
+    return gemm_f32(x, C_in, W, C_out, 0, y, C_out, B, C_out, C_in, EPI_BIAS, ea, ST(stream));
+}
+int sd3_partial_linear(const float* x, const float* W, const float* b, float* y, int M, int K, int N, int Nmax, int n0, void* stream) {
+    SD3_REQUIRE(M >= 0 && K > 0 && N > 0 && n0 >= 0 && n0 + N <= Nmax, "partial_linear: bad sizes M=%d K=%d N=%d Nmax=%d n0=%d", M, K, N, Nmax, n0);
+    if (M == 0) return SD3_OK;
+    NOTNULL(x); NOTNULL(W); NOTNULL(b); NOTNULL(y);
+    GemmEpilogueArgs ea;
+    ea.bias = b;
+    return gemm_f32(x, K, W, Nmax, n0, y, N, M, N, K, EPI_BIAS, ea, ST(stream));
+}
+int sd3_add(const float* a, const float* b, float* out, long long n, void* stream) {
+    SD3_REQUIRE(n >= 0, "add: negative size");
+    if (n == 0) return SD3_OK;
+    NOTNULL(a); NOTNULL(b); NOTNULL(out);
+    return add_op(a, b, out, n, ST(stream));
+}
+int sd3_multihead_attention(const float* Q, const float* K, const float* V, float* out, int B, int num_heads, int T, int L, int head_dim, void* stream) {
+    SD3_REQUIRE(B >= 0 && num_heads > 0 && T >= 0 && L > 0 && head_dim > 0, "multihead_attention: bad sizes B=%d heads=%d T=%d L=%d head_dim=%d", B,
+                num_heads, T, L, head_dim);
+    if (B == 0 || T == 0) return SD3_OK;
+    NOTNULL(Q); NOTNULL(K); NOTNULL(V); NOTNULL(out);
+    AttnSegments a{};
+    const int C = num_heads * head_dim;
+    a.q[0] = Q; a.k[0] = K; a.v[0] = V; a.out[0] = out;
+    a.ld_qkv[0] = a.ld_qkv[1] = C; a.ld_out[0] = a.ld_out[1] = C;
+    a.T[0] = L; a.Tq[0] = T;
+    return attention_f32(a, B, num_heads, head_dim, ST(stream));
+}
+int sd3_sinusoidal_embedding(const float* timesteps, float* out, int B, int emb_dim, void* stream) {
+    SD3_REQUIRE(B >= 0 && emb_dim > 0 && emb_dim % 2 == 0, "sinusoidal_embedding: bad sizes B=%d emb_dim=%d", B, emb_dim);
+    if (B == 0) return SD3_OK;
+    NOTNULL(timesteps); NOTNULL(out);
+    return timestep_embedding(timesteps, out, B, emb_dim, ST(stream));
+}
+int sd3_positional_embedding2D(float* out, int emb_dim, int height, int width, int base_size, void* stream) {
+    SD3_REQUIRE(emb_dim > 0 && emb_dim % 4 == 0 && height > 0 && width > 0, "positional_embedding2D: bad sizes emb_dim=%d height=%d width=%d", emb_dim,
+                height, width);
+    NOTNULL(out);
+    return pos_embed_table(out, emb_dim, height, width, base_size, ST(stream));
+}
+int sd3_crop_positional_embedding2D(const float* pos_embed, float* out, int pos_embed_max_size, int new_height, int new_width, int emb_dim, void* stream) {
+    SD3_REQUIRE(new_height > 0 && new_width > 0 && emb_dim > 0 && new_height <= pos_embed_max_size && new_width <= pos_embed_max_size,
+                "crop_positional_embedding2D: %dx%d does not fit a table of size %d", new_height, new_width, pos_embed_max_size);
+    NOTNULL(pos_embed); NOTNULL(out);
+    return pos_embed_crop(pos_embed, out, pos_embed_max_size, new_height, new_width, emb_dim, ST(stream));
+}
+int sd3_conv2d(const float* in, float* out, const float* kernel, const float* bias, int B, int kernel_height, int kernel_width, int in_channels,
+               int out_channels, int in_height, int in_width, int out_height, int out_width, int stride, int padding, void* stream) {
+    SD3_REQUIRE(B >= 0 && kernel_height > 0 && kernel_width > 0 && in_channels > 0 && out_channels > 0 && stride > 0 && padding >= 0, "conv2d: bad sizes");
+    SD3_REQUIRE(out_height == (in_height + 2 * padding - kernel_height) / stride + 1 && out_width == (in_width + 2 * padding - kernel_width) / stride + 1,
+                "conv2d: output size %dx%d does not match the input/kernel/stride/padding", out_height, out_width);
+    if (B == 0) return SD3_OK;
+    NOTNULL(in); NOTNULL(out); NOTNULL(kernel); NOTNULL(bias);
+    return conv2d_direct(in, out, kernel, bias, B, kernel_height, kernel_width, in_channels, out_channels, in_height, in_width, out_height, out_width,
+                         stride, padding, ST(stream));
+}
+int sd3_patch_embedding(const float* latent, float* out, const float* kernel, const float* bias, int B, int H, int W, int C_in, int emb_dim,
+                        int patch_size, int pos_embed_max_size, int base_height, void* stream) {
+    SD3_REQUIRE(B >= 0 && H > 0 && W > 0 && C_in > 0 && emb_dim > 0 && emb_dim % 4 == 0 && patch_size > 0, "patch_embedding: bad sizes");
+    const int hp = (H - patch_size) / patch_size + 1, wp = (W - patch_size) / patch_size + 1;
+    SD3_REQUIRE(hp > 0 && wp > 0 && hp <= pos_embed_max_size && wp <= pos_embed_max_size,
+                "patch_embedding: a %dx%d patch grid does not fit pos_embed_max_size=%d", hp, wp, pos_embed_max_size);
+    if (B == 0) return SD3_OK;
+    NOTNULL(latent); NOTNULL(out); NOTNULL(kernel); NOTNULL(bias);
+    return patch_embed_direct(latent, out, kernel, bias, B, H, W, C_in, emb_dim, patch_size, pos_embed_max_size, base_height, ST(stream));
+}
+int sd3_mlp(const float* x, float* out, float* h1, const float* W1, const float* b1, const float* W2, const float* b2, int B, int C_in, int C_hid,
+            int C_out, int activation, void* stream) {
+    SD3_REQUIRE(B >= 0 && C_in > 0 && C_hid > 0 && C_out > 0, "mlp: bad sizes");
+    SD3_REQUIRE(activation == SD3_ACT_SILU || activation == SD3_ACT_GELU_TANH, "mlp: unknown activation %d", activation);
+    if (B == 0) return SD3_OK;
+    NOTNULL(x); NOTNULL(out); NOTNULL(h1); NOTNULL(W1); NOTNULL(b1); NOTNULL(W2); NOTNULL(b2);
+    GemmEpilogueArgs ea;
+    ea.bias = b1;
+    SD3_TRY(gemm_f32(x, C_in, W1, C_hid, 0, h1, C_hid, B, C_hid, C_in, activation == SD3_ACT_SILU ? EPI_BIAS_SILU : EPI_BIAS_GELU, ea, ST(stream)));
+    ea.bias = b2;
+    return gemm_f32(h1, C_hid, W2, C_out, 0, out, C_out, B, C_out, C_hid, EPI_BIAS, ea, ST(stream));
+}
+int sd3_scale_and_shift(const float* in, float* out, const float* shift, const float* scale, int B, int T, int C, void* stream) {
+    SD3_REQUIRE(B >= 0 && T >= 0 && C > 0, "scale_and_shift: bad sizes");
+    if ((long long)B * T == 0) return SD3_OK;
+    NOTNULL(in); NOTNULL(out); NOTNULL(shift); NOTNULL(scale);
+    return modulate_op(in, out, shift, scale, B, T, C, ST(stream));
+}
+int sd3_gating_mechanism(const float* in, float* out, const float* gate, int B, int T, int C, void* stream) {
+    SD3_REQUIRE(B >= 0 && T >= 0 && C > 0, "gating_mechanism: bad sizes");
+    if ((long long)B * T == 0) return SD3_OK;
+    NOTNULL(in); NOTNULL(out); NOTNULL(gate);
+    return gate_op(in, out, gate, B, T, C, ST(stream));
+}
+int sd3_concatenate_along_tokens(const float* x, const float* y, float* out, int B, int Tx, int Ty, int C, void* stream) {
+    SD3_REQUIRE(B >= 0 && Tx >= 0 && Ty >= 0 && C > 0, "concatenate_along_tokens: bad sizes");
+    if (B == 0) return SD3_OK;
+    NOTNULL(out);
+    const long long T = (long long)Tx + Ty;
+    if (Tx) { NOTNULL(x); SD3_TRY(copy_rows(x, (long long)Tx * C, out, T * C, B, (long long)Tx * C, ST(stream))); }
+    if (Ty) { NOTNULL(y); SD3_TRY(copy_rows(y, (long long)Ty * C, out + (long long)Tx * C, T * C, B, (long long)Ty * C, ST(stream))); }
+    return SD3_OK;
+}
+int sd3_split_along_tokens(const float* in, float* split1, float* split2, int B, int T1, int T2, int C, void* stream) {
+    SD3_REQUIRE(B >= 0 && T1 >= 0 && T2 >= 0 && C > 0, "split_along_tokens: bad sizes");
+    if (B == 0) return SD3_OK;
+    NOTNULL(in);
+    const long long T = (long long)T1 + T2;
+    if (T1) { NOTNULL(split1); SD3_TRY(copy_rows(in, T * C, split1, (long long)T1 * C, B, (long long)T1 * C, ST(stream))); }
+    if (T2) { NOTNULL(split2); SD3_TRY(copy_rows(in + (long long)T1 * C, T * C, split2, (long long)T2 * C, B, (long long)T2 * C, ST(stream))); }
+    return SD3_OK;
+}
+
+// ------------------------------------------------------------------ context
+int sd3_ctx_create(sd3_ctx** out, int device) {
+    NOTNULL(out);
+    *out = nullptr;
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess || n == 0) {
+        (void)hipGetLastError();
+        return fail(SD3_ERR_HIP, "no HIP device available (%s)", e == hipSuccess ? "device count is 0" : hipGetErrorString(e));
+    }
+    SD3_REQUIRE(device >= 0 && device < n, "ctx_create: device %d out of range (0..%d)", device, n - 1);
+    sd3_ctx* c = new (std::nothrow) sd3_ctx();
+    if (!c) return fail(SD3_ERR_OOM, "ctx_create: out of host memory");
+    c->device = device;
+    *out = c;
+    return SD3_OK;
+}
+int sd3_weights_clear(sd3_ctx* ctx) {
+    NOTNULL(ctx);
+    DeviceGuard g(ctx->device);
+    SD3_HIP_TRY(hipStreamSynchronize(ctx->stream));
+    for (auto& kv : ctx->packed) (void)hipFree(kv.second.ptr);
+    ctx->packed.clear();
+    ctx->params.clear();
+    return SD3_OK;
+}
+int sd3_ctx_destroy(sd3_ctx* ctx) {
+    if (!ctx) return SD3_OK;
+    {
+        DeviceGuard g(ctx->device);
+        (void)hipStreamSynchronize(ctx->stream);
+        for (auto& kv : ctx->packed) (void)hipFree(kv.second.ptr);
+        for (auto& kv : ctx->pos_tables) (void)hipFree(kv.second);
+        if (ctx->ws) (void)hipFree(ctx->ws);
+        (void)hipGetLastError();
+    }
+    delete ctx;
+    return SD3_OK;
+}
+int sd3_ctx_set_stream(sd3_ctx* ctx, void* stream) {
+    NOTNULL(ctx);
+    ctx->stream = ST(stream);
+    return SD3_OK;
+}
+int sd3_ctx_synchronize(sd3_ctx* ctx) {
+    NOTNULL(ctx);
+    DeviceGuard g(ctx->device);
+    SD3_HIP_TRY(hipStreamSynchronize(ctx->stream));
+    return SD3_OK;
+}
+int sd3_weights_bind(sd3_ctx* ctx, const char* name, const float* ptr, long long numel) {
+    NOTNULL(ctx); NOTNULL(name); NOTNULL(ptr);
+    SD3_REQUIRE(numel > 0, "weights_bind(%s): numel must be positive", name);
+    SD3_REQUIRE((reinterpret_cast<uintptr_t>(ptr) & 3) == 0, "weights_bind(%s): pointer is not 4-byte aligned", name);
+    ctx->params[name] = std::make_pair(ptr, numel);
+    return SD3_OK;
+}
+int sd3_weights_prepare(sd3_ctx* ctx, int precision) {
+    NOTNULL(ctx);
+    SD3_REQUIRE(precision == SD3_PREC_F32 || precision == SD3_PREC_BF16, "weights_prepare: unknown precision %d", precision);
+    // Drop stale copies; they are rebuilt from the bound fp32 tensors on next use.
+    DeviceGuard g(ctx->device);
+    SD3_HIP_TRY(hipStreamSynchronize(ctx->stream));
+    for (auto& kv : ctx->packed) (void)hipFree(kv.second.ptr);
+    ctx->packed.clear();
+    return SD3_OK;
+}
+
+// ------------------------------------------------------------------ block
+int sd3_dit_block_w(sd3_ctx* ctx, const float* y, float* c, float* x, const sd3_block_weights* w, int B, int Tc, int Tx, int emb_dim, int attn_heads,
+                    int mlp_expand, int use_dual_attention, int use_qk_norm, int discard_context, int precision) {
+    NOTNULL(ctx); NOTNULL(y); NOTNULL(x); NOTNULL(w);
+    SD3_REQUIRE(attn_heads > 0, "block: attn_heads must be positive");
+    Dims d{B, Tc, Tx, emb_dim, attn_heads, emb_dim / attn_heads, mlp_expand, use_dual_attention != 0, use_qk_norm != 0, discard_context != 0};
+    SD3_TRY(check_block_dims(d, precision));
+    if (Tc > 0) NOTNULL(c);
+    DeviceGuard g(ctx->device);
+    if (!g.ok) return fail(SD3_ERR_HIP, "cannot select device %d", ctx->device);
+    SD3_TRY(ensure_workspace(ctx, block_workspace_bytes(d, precision)));
+    Bump ws(ctx->ws, ctx->ws_bytes);
+    return run_block(ctx, precision, y, c, x, *w, d, nullptr, nullptr, ws);
+}
+
+int sd3_dit_block(sd3_ctx* ctx, const float* y, float* c, float* x, const char* prefix, int B, int Tc, int Tx, int emb_dim, int attn_heads, int mlp_expand,
+                  int use_dual_attention, int use_qk_norm, int discard_context, int precision) {
+    NOTNULL(ctx);
+    SD3_REQUIRE(attn_heads > 0 && emb_dim > 0, "block: emb_dim and attn_heads must be positive");
+    Dims d{B, Tc, Tx, emb_dim, attn_heads, emb_dim / attn_heads, mlp_expand, use_dual_attention != 0, use_qk_norm != 0, discard_context != 0};
+    SD3_TRY(check_block_dims(d, precision));
+    sd3_block_weights w;
+    SD3_TRY(lookup_block_weights(ctx, prefix ? prefix : "", d, &w));
+    return sd3_dit_block_w(ctx, y, c, x, &w, B, Tc, Tx, emb_dim, attn_heads, mlp_expand, use_dual_attention, use_qk_norm, discard_context, precision);
+}
+
+// ------------------------------------------------------------------ full forward
+int sd3_dit_forward(sd3_ctx* ctx, const float* pooled, const float* captions, const float* latent, const float* timesteps, float* out, int B, int Tc,
+                    int H, int W, int num_layers, const int* dual_attention_layers, int n_dual, int pooled_dim, int captions_dim, int C_in, int emb_dim,
+                    int attn_heads, int mlp_expand, int patch_size, int pos_embed_max_size, int base_height, int use_qk_norm, int precision) {
+    NOTNULL(ctx); NOTNULL(pooled); NOTNULL(captions); NOTNULL(latent); NOTNULL(timesteps); NOTNULL(out);
+    SD3_REQUIRE(num_layers > 0 && patch_size > 0 && H >= patch_size && W >= patch_size && C_in > 0 && pooled_dim > 0 && captions_dim > 0 && attn_heads > 0 &&
+                    emb_dim > 0 && n_dual >= 0 && (n_dual == 0 || dual_attention_layers),
+                "DiT: bad sizes");
+    const int C = emb_dim, p = patch_size;
+    const int Hp = (H - p) / p + 1, Wp = (W - p) / p + 1, Tx = Hp * Wp, PPC = p * p * C_in, Kp = C_in * p * p;
+    SD3_REQUIRE(Hp <= pos_embed_max_size && Wp <= pos_embed_max_size, "DiT: a %dx%d patch grid does not fit pos_embed_max_size=%d", Hp, Wp, pos_embed_max_size);
+    SD3_REQUIRE(C % 4 == 0, "DiT: emb_dim must be a multiple of 4");
+    Dims dmax{B, Tc, Tx, C, attn_heads, C / attn_heads, mlp_expand, n_dual > 0, use_qk_norm != 0, false};
+    SD3_TRY(check_block_dims(dmax, precision));
+    const bool bf = precision == SD3_PREC_BF16;
+    if (bf && ((captions_dim % 64) || (Kp % 64))) return fail(SD3_ERR_UNSUPPORTED, "bf16 path needs captions_dim and C_in*patch^2 to be multiples of 64");
+    DeviceGuard g(ctx->device);
+    if (!g.ok) return fail(SD3_ERR_HIP, "cannot select device %d", ctx->device);
+    hipStream_t st = ctx->stream;
+
+    std::vector<char> is_dual(num_layers, 0);
+    for (int i = 0; i < n_dual; i++)
+        if (dual_attention_layers[i] >= 0 && dual_attention_layers[i] < num_layers) is_dual[dual_attention_layers[i]] = 1;
+
+    // ---- weights by name (modules.cpp:1665-1728)
+    int pst = SD3_OK;
+    auto P = [&](const char* n, long long numel) -> const float* {
+        const float* q = find_param(ctx, n, numel, &pst);
+        if (!q && pst == SD3_OK) pst = fail(SD3_ERR_MISSING_PARAM, "parameter %s is not bound", n);
+        return q;
+    };
+    const float* t_w0 = P("timestep_mlp.0.weight", 256LL * C); const float* t_b0 = P("timestep_mlp.0.bias", C);
+    const float* t_w2 = P("timestep_mlp.2.weight", (long long)C * C); const float* t_b2 = P("timestep_mlp.2.bias", C);
+    const float* p_w0 = P("pooled_mlp.0.weight", (long long)pooled_dim * C); const float* p_b0 = P("pooled_mlp.0.bias", C);
+    const float* p_w2 = P("pooled_mlp.2.weight", (long long)C * C); const float* p_b2 = P("pooled_mlp.2.bias", C);
+    const float* cap_w = P("captions_linear.weight", (long long)captions_dim * C); const float* cap_b = P("captions_linear.bias", C);
+    const float* patch_w = P("to_patch.conv.weight", (long long)C * Kp); const float* patch_b = P("to_patch.conv.bias", C);
+    const float* ao_w = P("ada_ln_out.linear.weight", 2LL * C * C); const float* ao_b = P("ada_ln_out.linear.bias", 2LL * C);
+    const float* out_w = P("linear_out.weight", (long long)C * PPC); const float* out_b = P("linear_out.bias", PPC);
+    if (pst != SD3_OK) return pst;
+    std::vector<sd3_block_weights> bw(num_layers);
+    std::vector<Dims> bd(num_layers, dmax);
+    for (int l = 0; l < num_layers; l++) {
+        bd[l].dual = is_dual[l] != 0;
+        bd[l].discard = (l == num_layers - 1);
+        SD3_TRY(lookup_block_weights(ctx, "transformer." + std::to_string(l) + ".", bd[l], &bw[l]));
+        if (!bw[l].c_ada_w || !bw[l].c_ada_b || !bw[l].x_ada_w || !bw[l].x_ada_b)
+            return fail(SD3_ERR_MISSING_PARAM, "transformer.%d: adaLN modulation weights are not bound", l);
+    }
+
+    // ---- workspace
+    auto layout = [&](Bump& b, float** temb, float** h1, float** yt, float** yp, float** y, float** c, float** x, void** cap_in, void** patches,
+                      float** ada_all, float** ada_out, float** tokens) {
+        *temb = b.take<float>((size_t)B * 256);
+        *h1 = b.take<float>((size_t)B * C);
+        *yt = b.take<float>((size_t)B * C);
+        *yp = b.take<float>((size_t)B * C);
+        *y = b.take<float>((size_t)B * C);
+        *c = b.take<float>((size_t)B * Tc * C);
+        *x = b.take<float>((size_t)B * Tx * C);
+        *cap_in = bf ? (void*)b.take<bf16_t>((size_t)B * Tc * captions_dim) : nullptr;
+        *patches = b.take<char>((size_t)B * Tx * Kp * (bf ? 2 : 4));
+        *ada_all = b.take<float>((size_t)B * 15 * C * num_layers);
+        *ada_out = b.take<float>((size_t)B * 2 * C);
+        *tokens = b.take<float>((size_t)B * Tx * PPC);
+    };
+    float *temb, *h1, *yt, *yp, *y, *c, *x, *ada_all, *ada_out, *tokens;
+    void *cap_in, *patches;
+    Bump probe(nullptr, 0);
+    layout(probe, &temb, &h1, &yt, &yp, &y, &c, &x, &cap_in, &patches, &ada_all, &ada_out, &tokens);
+    SD3_TRY(ensure_workspace(ctx, probe.off + block_workspace_bytes(dmax, precision)));
+    Bump ws(ctx->ws, ctx->ws_bytes);
+    layout(ws, &temb, &h1, &yt, &yp, &y, &c, &x, &cap_in, &patches, &ada_all, &ada_out, &tokens);
+    const size_t block_ws_off = ws.off;
+
+    // ---- y = silu(MLP(t_emb) + MLP(pooled)) (modules.cpp:1663-1675); weights stay fp32 here: 8 MB read once
+    SD3_TRY(timestep_embedding(timesteps, temb, B, 256, st));
+    {
+        SmallLinearJob j1{t_w0, t_b0, h1, C, C, 0};
+        SD3_TRY(small_linear_batched(temb, B, 256, &j1, 1, 0, SD3_ACT_SILU, st));
+        SmallLinearJob j2{t_w2, t_b2, yt, C, C, 0};
+        SD3_TRY(small_linear_batched(h1, B, C, &j2, 1, 0, -1, st));
+        SmallLinearJob j3{p_w0, p_b0, h1, C, C, 0};
+        SD3_TRY(small_linear_batched(pooled, B, pooled_dim, &j3, 1, 0, SD3_ACT_SILU, st));
+        SmallLinearJob j4{p_w2, p_b2, yp, C, C, 0};
+        SD3_TRY(small_linear_batched(h1, B, C, &j4, 1, 0, -1, st));
+        SD3_TRY(add_silu_op(yt, yp, y, (long long)B * C, st));
+    }
+    // ---- c = captions @ W + b (modules.cpp:1678)
+    {
+        GemmEpilogueArgs none;
+        const void* a_in = captions;
+        if (bf) {
+            SD3_TRY(cast_f32_to_bf16(captions, (bf16_t*)cap_in, (long long)B * Tc * captions_dim, st));
+            a_in = cap_in;
+        }
+        if (Tc > 0) SD3_TRY(linear_layer(ctx, precision, a_in, cap_w, cap_b, c, 1, C, B * Tc, C, captions_dim, EPI_BIAS, none));
+    }
+    // ---- x = patchify-conv(latent) + bias + position table (modules.cpp:1682 -> 1093-1117) as an im2col GEMM
+    {
+        auto key = std::make_tuple(C, pos_embed_max_size, base_height / p, Hp, Wp);
+        float* table = nullptr;
+        auto it = ctx->pos_tables.find(key);
+        if (it == ctx->pos_tables.end()) {
+            hipError_t e = hipMalloc((void**)&table, (size_t)Tx * C * sizeof(float));
+            if (e != hipSuccess) {
+                (void)hipGetLastError();
+                return fail(SD3_ERR_OOM, "position table: %s", hipGetErrorString(e));
+            }
+            int rc = pos_embed_cropped(table, C, pos_embed_max_size, base_height / p, Hp, Wp, st);
+            if (rc != SD3_OK) {
+                (void)hipFree(table);
+                return rc;
+            }
+            ctx->pos_tables[key] = table;
+        } else {
+            table = it->second;
+        }
+        SD3_TRY(im2col_patches(latent, patches, bf, B, C_in, H, W, p, st));
+        GemmEpilogueArgs ea;
+        ea.bias = patch_b; ea.table = table; ea.rows_per_batch = Tx;
+        if (bf) {
+            // the conv weight (C, C_in*p*p) is already (N,K) K-contiguous: its MFMA form is a plain cast
+            const void* wp = nullptr;
+            SD3_TRY(get_packed(ctx, patch_w, C, Kp, 1, &wp));
+            SD3_TRY(gemm_bf16((const bf16_t*)patches, (const bf16_t*)wp, x, 1, C, B * Tx, C, Kp, EPI_BIAS_ROWADD, ea, st));
+        } else {
+            const void* wt = nullptr;
+            SD3_TRY(get_packed(ctx, patch_w, Kp, C, 2, &wt));
+            SD3_TRY(gemm_f32((const float*)patches, Kp, (const float*)wt, C, 0, x, C, B * Tx, C, Kp, EPI_BIAS_ROWADD, ea, st));
+        }
+    }
+    // ---- modulation vectors of every block and of the output layer: y does not change across blocks, so all
+    //      adaLN projections (0.77 G parameters) are streamed once, up front
+    {
+        std::vector<SmallLinearJob> jobs;
+        for (int l = 0; l < num_layers; l++) {
+            const int cch = bd[l].discard ? 2 : 6, xch = bd[l].dual ? 9 : 6;
+            float* base = ada_all + (size_t)l * B * 15 * C;
+            jobs.push_back({bw[l].c_ada_w, bw[l].c_ada_b, base, cch * C, cch * C, 0});
+            jobs.push_back({bw[l].x_ada_w, bw[l].x_ada_b, base + (size_t)B * 6 * C, xch * C, xch * C, 0});
+        }
+        jobs.push_back({ao_w, ao_b, ada_out, 2 * C, 2 * C, 0});
+        SD3_TRY(ada_jobs_run(ctx, precision, y, B, C, jobs));
+    }
+    // ---- blocks (modules.cpp:1687-1718)
+    for (int l = 0; l < num_layers; l++) {
+        Bump bws(ctx->ws, ctx->ws_bytes);
+        bws.off = block_ws_off;
+        const float* base = ada_all + (size_t)l * B * 15 * C;
+        SD3_TRY(run_block(ctx, precision, y, c, x, bw[l], bd[l], base, base + (size_t)B * 6 * C, bws));
+    }
+    // ---- output layer: LN(eps 1e-5), chunk 0 = scale, chunk 1 = shift, projection, tokens -> pixels (modules.cpp:1721-1752)
+    {
+        Bump bws(ctx->ws, ctx->ws_bytes);
+        bws.off = block_ws_off;
+        void* x_hid = bws.take<char>((size_t)B * Tx * C * (bf ? 2 : 4));
+        SD3_TRY(layernorm_modulate(x, x_hid, nullptr, ada_out + C, ada_out, nullptr, nullptr, 2 * C, 1e-5f, B, Tx, C, bf, st));
+        GemmEpilogueArgs none;
+        SD3_TRY(linear_layer(ctx, precision, x_hid, out_w, out_b, tokens, 1, PPC, B * Tx, PPC, C, EPI_BIAS, none));
+        SD3_TRY(unpatchify(tokens, out, B, C_in, H, W, p, st));
+    }
+    return SD3_OK;
+}
+
+// ------------------------------------------------------------------ bf16 kernels on their own
+int sd3_flash_attention_bf16(const void* qkv0, const void* qkv1, void* out0, void* out1, const float* rms_q0, const float* rms_k0, const float* rms_q1,
+                             const float* rms_k1, int B, int T0, int T1, int num_heads, int head_dim, void* stream) {
+    SD3_REQUIRE(B >= 0 && T0 >= 0 && T1 >= 0 && num_heads > 0 && head_dim > 0, "flash_attention_bf16: bad sizes");
+    if (B == 0 || T0 + T1 == 0) return SD3_OK;
+    const int C = num_heads * head_dim;
+    AttnSegments a{};
+    const void* qkv[2] = {qkv0, qkv1};
+    void* outs[2] = {out0, out1};
+    const float* rq[2] = {rms_q0, rms_q1};
+    const float* rk[2] = {rms_k0, rms_k1};
+    const int T[2] = {T0, T1};
+    for (int i = 0; i < 2; i++) {
+        if (T[i] > 0) SD3_REQUIRE(qkv[i] != nullptr, "flash_attention_bf16: null qkv buffer for segment %d", i);
+        a.q[i] = qkv[i];
+        a.k[i] = qkv[i] ? (const char*)qkv[i] + (size_t)C * 2 : nullptr;
+        a.v[i] = qkv[i] ? (const char*)qkv[i] + (size_t)2 * C * 2 : nullptr;
+        a.out[i] = outs[i];
+        a.ld_qkv[i] = 3 * C; a.ld_out[i] = C;
+        a.T[i] = a.Tq[i] = T[i];
+        a.rms_q[i] = rq[i]; a.rms_k[i] = rk[i];
+    }
+    return attention_bf16(a, B, num_heads, head_dim, ST(stream));
+}
+int sd3_pack_weight_bf16(const float* W, void* wpacked, int K, int N, void* stream) {
+    SD3_REQUIRE(K > 0 && N > 0, "pack_weight_bf16: bad sizes");
+    NOTNULL(W); NOTNULL(wpacked);
+    return pack_weight_bf16(W, (bf16_t*)wpacked, K, N, ST(stream));
+}
+int sd3_gemm_bf16(const void* A, const void* wpacked, const float* bias, void* out, int M, int N, int K, int epilogue, void* stream) {
+    SD3_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_bf16: bad sizes");
+    SD3_REQUIRE(epilogue == EPI_BIAS || epilogue == EPI_BIAS_GELU, "gemm_bf16: epilogue must be 0 (bias) or 1 (bias+GELU)");
+    if (M == 0) return SD3_OK;
+    NOTNULL(A); NOTNULL(wpacked); NOTNULL(out);
+    GemmEpilogueArgs ea;
+    ea.bias = bias;
+    return gemm_bf16((const bf16_t*)A, (const bf16_t*)wpacked, out, 0, N, M, N, K, epilogue, ea, ST(stream));
+}
+int sd3_cast_f32_to_bf16(const float* in, void* out, long long n, void* stream) {
+    SD3_REQUIRE(n >= 0, "cast: negative size");
+    if (n == 0) return SD3_OK;
+    NOTNULL(in); NOTNULL(out);
+    return cast_f32_to_bf16(in, (bf16_t*)out, n, ST(stream));
+}
+
+}  // extern "C"

@@ -1,0 +1,143 @@
+// Linear layers whose left operand has at most 8 rows (the batch): the adaLN modulation projections
+// (modules.cpp:1384-1501 compute them one 1536-column chunk at a time with partial_linear), the timestep and
+// pooled-text MLPs (modules.cpp:1664-1671). They are pure weight streaming, so one launch covers a whole list
+// of weight matrices ("jobs") and reads every weight element exactly once, N-contiguous as the reference stores it.
+#include "common.hpp"
+
+namespace sd3 {
+
+template <typename WT>
+struct WLoad;
+template <>
+struct WLoad<float> {
+    static __device__ __forceinline__ void load4(const float* p, float (&w)[4]) {
+        float4 v = *reinterpret_cast<const float4*>(p);
+        w[0] = v.x; w[1] = v.y; w[2] = v.z; w[3] = v.w;
+    }
+    static __device__ __forceinline__ float load1(const float* p) { return *p; }
+};
+template <>
+struct WLoad<bf16_t> {
+    static __device__ __forceinline__ void load4(const bf16_t* p, float (&w)[4]) {
+        uint2 v = *reinterpret_cast<const uint2*>(p);
+        w[0] = __uint_as_float(v.x << 16); w[1] = __uint_as_float(v.x & 0xffff0000u);
+        w[2] = __uint_as_float(v.y << 16); w[3] = __uint_as_float(v.y & 0xffff0000u);
+    }
+    static __device__ __forceinline__ float load1(const bf16_t* p) { return bf16_to_f32(*p); }
+};
+
+// Block = 256 threads = 32 column groups (4 columns each, 128 columns per block) x 8 slices of K.
+// x is staged transposed in LDS (xs[k][m]) so that a thread reads its M inputs for one k with wide LDS loads.
+// Jobs travel as a kernel argument (no device-side table to keep coherent with the host).
+struct SmallLinearJobPack {
+    SmallLinearJob j[16];
+};
+
+template <int M, typename WT, bool VEC>
+__global__ void __launch_bounds__(256) small_linear_kernel(const float* __restrict__ x, int m_real, int K, const SmallLinearJobPack jobs, int act) {
+    extern __shared__ float smem[];
+    const SmallLinearJob job = jobs.j[blockIdx.y];
+    const int col_base = blockIdx.x * 128;
+    if (col_base >= job.N) return;
+    const int tid = threadIdx.x;
+    for (int idx = tid; idx < M * K; idx += 256) {
+        const int m = idx / K, k = idx - m * K;
+        smem[k * M + m] = (m < m_real) ? x[(long long)m * K + k] : 0.f;
+    }
+    __syncthreads();
+
+    const int cl = tid & 31, ks = tid >> 5;
+    const int c0 = col_base + cl * 4;
+    const int kper = (K + 7) / 8;
+    const int kbeg = ks * kper, kend = min(K, kbeg + kper);
+    const WT* W = reinterpret_cast<const WT*>(job.W) + job.n0 + c0;
+    float acc[M][4];
+#pragma unroll
+    for (int m = 0; m < M; m++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) acc[m][j] = 0.f;
+
+    if (c0 < job.N) {
+#pragma unroll 4
+        for (int k = kbeg; k < kend; k++) {
+            float w[4];
+            if (VEC) {
+                WLoad<WT>::load4(W + (long long)k * job.ldw, w);
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; j++) w[j] = (c0 + j < job.N) ? WLoad<WT>::load1(W + (long long)k * job.ldw + j) : 0.f;
+            }
+#pragma unroll
+            for (int m = 0; m < M; m++) {
+                const float xv = smem[k * M + m];
+#pragma unroll
+                for (int j = 0; j < 4; j++) acc[m][j] += xv * w[j];
+            }
+        }
+    }
+    __syncthreads();  // everyone is done with xs; reuse it for the cross-slice reduction: red[ks][m][128]
+#pragma unroll
+    for (int m = 0; m < M; m++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) smem[(ks * M + m) * 128 + cl * 4 + j] = acc[m][j];
+    __syncthreads();
+    for (int e = tid; e < M * 128; e += 256) {
+        const int m = e >> 7, c = e & 127;
+        const int col = col_base + c;
+        if (m < m_real && col < job.N) {
+            float s = 0.f;
+#pragma unroll
+            for (int s8 = 0; s8 < 8; s8++) s += smem[(s8 * M + m) * 128 + c];
+            if (job.bias) s += job.bias[job.n0 + col];
+            if (act == SD3_ACT_SILU) s = silu_precise(s);
+            else if (act == SD3_ACT_GELU_TANH) s = gelu_tanh_precise(s);
+            job.out[(long long)m * job.N + col] = s;
+        }
+    }
+}
+
+template <int M>
+static void launch_small(const float* x, int m_real, int K, const SmallLinearJobPack& jobs, int n_jobs, int max_N, int w_is_bf16, bool vec, int act,
+                         hipStream_t st) {
+    dim3 grid((max_N + 127) / 128, n_jobs), block(256);
+    const int kk = K > 1024 ? K : 1024;
+    const size_t smem = (size_t)kk * M * sizeof(float);
+    if (w_is_bf16) {
+        if (vec) hipLaunchKernelGGL((small_linear_kernel<M, bf16_t, true>), grid, block, smem, st, x, m_real, K, jobs, act);
+        else hipLaunchKernelGGL((small_linear_kernel<M, bf16_t, false>), grid, block, smem, st, x, m_real, K, jobs, act);
+    } else {
+        if (vec) hipLaunchKernelGGL((small_linear_kernel<M, float, true>), grid, block, smem, st, x, m_real, K, jobs, act);
+        else hipLaunchKernelGGL((small_linear_kernel<M, float, false>), grid, block, smem, st, x, m_real, K, jobs, act);
+    }
+}
+
+int small_linear_batched(const float* x, int M, int K, const SmallLinearJob* jobs_host, int n_jobs, int w_is_bf16, int act, hipStream_t st) {
+    if (M <= 0 || n_jobs <= 0) return SD3_OK;
+    if (M > 8) return fail(SD3_ERR_UNSUPPORTED, "small_linear: at most 8 rows (got %d)", M);
+    if ((size_t)(K > 1024 ? K : 1024) * 8 * sizeof(float) > 65536 && M > 4)
+        return fail(SD3_ERR_UNSUPPORTED, "small_linear: K=%d too large for %d rows", K, M);
+    if (K > 4096) return fail(SD3_ERR_UNSUPPORTED, "small_linear: K=%d too large", K);
+    const int esz = w_is_bf16 ? 2 : 4;
+    for (int base = 0; base < n_jobs; base += 16) {
+        const int n = (n_jobs - base) < 16 ? (n_jobs - base) : 16;
+        SmallLinearJobPack pack;
+        int max_N = 0;
+        bool vec = true;
+        for (int i = 0; i < n; i++) {
+            pack.j[i] = jobs_host[base + i];
+            const SmallLinearJob& j = pack.j[i];
+            if (j.N > max_N) max_N = j.N;
+            if ((j.N % 4) || (j.ldw % 4) || (j.n0 % 4) || ((reinterpret_cast<uintptr_t>(j.W) % (4 * esz)) != 0)) vec = false;
+        }
+        for (int i = n; i < 16; i++) pack.j[i] = SmallLinearJob{nullptr, nullptr, nullptr, 0, 0, 0};
+        if (max_N == 0) continue;
+        if (M == 1) launch_small<1>(x, M, K, pack, n, max_N, w_is_bf16, vec, act, st);
+        else if (M == 2) launch_small<2>(x, M, K, pack, n, max_N, w_is_bf16, vec, act, st);
+        else if (M <= 4) launch_small<4>(x, M, K, pack, n, max_N, w_is_bf16, vec, act, st);
+        else launch_small<8>(x, M, K, pack, n, max_N, w_is_bf16, vec, act, st);
+        SD3_TRY(launch_status("small_linear"));
+    }
+    return SD3_OK;
+}
+
+}  // namespace sd3

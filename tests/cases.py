@@ -31,6 +31,24 @@ DIT_CASES = {
 }
 
 
+# The configuration of the reference's own full-model check (module_tests/DiT.py:8-21): too slow for the CPU oracle
+# inside a test run, so its golden output is only compared with the GPU fp32 path.
+DIT_REFERENCE_TEST = ("dit_reference_test", DiTConfig(num_layers=3, dual_attention_layers=(0,), pooled_dim=2048, captions_dim=2048, in_channels=16,
+                                                      emb_dim=256, attn_heads=2, mlp_expand=4, patch_size=2, pos_embed_max_size=96, base_height=64,
+                                                      use_qk_norm=True), 2, 154, 64, 64)
+
+
+def dit_reference_test_case():
+    name, cfg, B, Tc, H, W = DIT_REFERENCE_TEST
+    rng = np.random.Generator(np.random.Philox(_seed(name)))
+    params = synthetic_params_numpy(dit_param_shapes(cfg), _seed(name) + 1, 0.05, 0.05)
+    latent = rng.standard_normal((B, cfg.in_channels, H, W), dtype=np.float32)
+    captions = rng.standard_normal((B, Tc, cfg.captions_dim), dtype=np.float32)
+    pooled = rng.standard_normal((B, cfg.pooled_dim), dtype=np.float32)
+    timesteps = rng.random((B,), dtype=np.float32)  # the reference draws timesteps from U[0,1) (module_tests/DiT.py:38)
+    return dict(cfg=cfg, latent=latent, captions=captions, pooled=pooled, timesteps=timesteps, params=params)
+
+
 def _seed(name):
     return 0x5D3 + sum(ord(ch) * (i + 1) for i, ch in enumerate(name))
 

@@ -27,6 +27,11 @@ def main():
         k = cases.dit_case(name)
         out[name + ".out"] = ol.ref_dit_forward(k["pooled"], k["captions"], k["latent"], k["timesteps"], k["params"], k["cfg"])
     np.savez_compressed(os.path.join(HERE, "reference_outputs.npz"), **out)
+    if "--with-reference-test-config" in sys.argv:  # about a minute of single-core CPU
+        k = cases.dit_reference_test_case()
+        big = ol.ref_dit_forward(k["pooled"], k["captions"], k["latent"], k["timesteps"], k["params"], k["cfg"])
+        np.savez_compressed(os.path.join(HERE, "reference_dit_test_config.npz"), out=big.astype(np.float32))
+        out["dit_reference_test.out"] = big
     for k, v in out.items():
         print(f"{k:28s} {str(v.shape):18s} absmax {np.abs(v).max():.4f}")
 

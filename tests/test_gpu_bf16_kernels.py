@@ -1,0 +1,92 @@
+"""The two MFMA kernels of the bf16 path on their own, against fp32 torch arithmetic on the bf16-rounded inputs."""
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import M, host, rel_l2
+from sd3_c_amd import lib as L
+
+pytestmark = pytest.mark.gpu
+
+
+def _naive_joint_attention(qkv0, qkv1, rq, rk, B, T0, T1, NH, HS):
+    """fp32 softmax(QK^T/8)V over [segment 0 ; segment 1] with per-head RMSNorm (eps 1e-6) of q and k, from bf16-rounded inputs."""
+    C = NH * HS
+
+    def split(qkv, T, wq, wk):
+        q, k, v = qkv.float().view(B, T, 3, NH, HS).unbind(2)
+
+        def rms(a, w):
+            return a * torch.rsqrt(a.pow(2).mean(-1, keepdim=True) + 1e-6) * w
+
+        return rms(q, wq), rms(k, wk), v
+
+    q0, k0, v0 = split(qkv0, T0, rq[0], rk[0])
+    parts = [(q0, k0, v0)]
+    if T1:
+        parts.append(split(qkv1, T1, rq[1], rk[1]))
+    q, k, v = (torch.cat([p[i] for p in parts], 1).transpose(1, 2) for i in range(3))  # (B,NH,T,HS)
+    out = torch.empty_like(q)
+    for b in range(B):
+        for h0 in range(0, NH, 4):
+            s = q[b, h0:h0 + 4] @ k[b, h0:h0 + 4].transpose(-1, -2) / 8.0
+            out[b, h0:h0 + 4] = torch.softmax(s, -1) @ v[b, h0:h0 + 4]
+    return out.transpose(1, 2).reshape(B, T0 + T1, C)
+
+
+@pytest.mark.parametrize("B,T0,T1,NH", [(2, 154, 4096, 24), (1, 154, 1024, 24), (2, 7, 130, 4), (1, 0 + 64, 0, 2), (1, 1, 63, 3)])
+def test_flash_attention_bf16(B, T0, T1, NH):
+    """BASELINE config 2 is the first case: B=2, 24 heads of 64, 154 text + 4096 image tokens, q/k/v ~ N(0,1)."""
+    HS, C = 64, NH * 64
+    g = torch.Generator(device="cuda").manual_seed(T0 * 7 + T1)
+    qkv0 = torch.randn((B * T0, 3 * C), device="cuda", generator=g).bfloat16()
+    qkv1 = torch.randn((B * max(T1, 1), 3 * C), device="cuda", generator=g).bfloat16()
+    rq = [1 + 0.1 * torch.randn(HS, device="cuda", generator=g) for _ in range(2)]
+    rk = [1 + 0.1 * torch.randn(HS, device="cuda", generator=g) for _ in range(2)]
+    out0 = torch.zeros((B * T0, C), device="cuda", dtype=torch.bfloat16)
+    out1 = torch.zeros((B * max(T1, 1), C), device="cuda", dtype=torch.bfloat16)
+    L.call("sd3_flash_attention_bf16", qkv0.data_ptr(), qkv1.data_ptr() if T1 else None, out0.data_ptr(), out1.data_ptr() if T1 else None,
+           rq[0].data_ptr(), rk[0].data_ptr(), rq[1].data_ptr(), rk[1].data_ptr(), B, T0, T1, NH, HS, None)
+    ref = _naive_joint_attention(qkv0, qkv1, rq, rk, B, T0, T1, NH, HS)
+    got = torch.cat([out0.view(B, T0, C)] + ([out1.view(B, T1, C)] if T1 else []), 1).float()
+    assert torch.isfinite(got).all()
+    assert rel_l2(host(got), host(ref)) <= 1e-2
+    assert float((got - ref).abs().max()) <= 0.05  # outputs are O(1) convex combinations of N(0,1) values
+
+
+def test_flash_attention_bf16_without_qk_norm_and_ones_v():
+    B, T0, T1, NH, HS = 1, 10, 200, 2, 64
+    C = NH * HS
+    qkv0 = torch.randn((B * T0, 3 * C), device="cuda").bfloat16()
+    qkv1 = torch.randn((B * T1, 3 * C), device="cuda").bfloat16()
+    qkv0[:, 2 * C:] = 1
+    qkv1[:, 2 * C:] = 1
+    out0 = torch.zeros((B * T0, C), device="cuda", dtype=torch.bfloat16)
+    out1 = torch.zeros((B * T1, C), device="cuda", dtype=torch.bfloat16)
+    L.call("sd3_flash_attention_bf16", qkv0.data_ptr(), qkv1.data_ptr(), out0.data_ptr(), out1.data_ptr(), None, None, None, None, B, T0, T1, NH, HS, None)
+    assert float((out0.float() - 1).abs().max()) <= 1e-2 and float((out1.float() - 1).abs().max()) <= 1e-2  # rows of softmax sum to one
+
+
+@pytest.mark.parametrize("Mr,N,K,epi", [(8192, 1536, 1536, 0), (308, 4608, 1536, 0), (1000, 6144, 1536, 1), (130, 64, 1536, 0), (257, 1536, 6144, 0), (5, 200, 64, 1)])
+def test_gemm_bf16(Mr, N, K, epi):
+    g = torch.Generator(device="cuda").manual_seed(Mr + N)
+    A = torch.randn((Mr, K), device="cuda", generator=g).bfloat16()
+    W = (0.05 * torch.randn((K, N), device="cuda", generator=g))
+    bias = torch.randn(N, device="cuda", generator=g)
+    Wp = torch.empty((N, K), device="cuda", dtype=torch.bfloat16)
+    L.call("sd3_pack_weight_bf16", W.data_ptr(), Wp.data_ptr(), K, N, None)
+    assert torch.equal(Wp, W.bfloat16().t().contiguous())
+    out = torch.empty((Mr, N), device="cuda", dtype=torch.bfloat16)
+    L.call("sd3_gemm_bf16", A.data_ptr(), Wp.data_ptr(), bias.data_ptr(), out.data_ptr(), Mr, N, K, epi, None)
+    ref = A.float() @ W.bfloat16().float() + bias
+    if epi == 1:
+        ref = torch.nn.functional.gelu(ref, approximate="tanh")
+    assert rel_l2(host(out), host(ref)) <= 5e-3  # bf16 rounding of the output is 2^-9 relative
+
+
+def test_cast_rounds_to_nearest_even():
+    x = torch.randn(100000, device="cuda") * 100
+    x[:4] = torch.tensor([0.0, -0.0, float("inf"), 1.00390625])  # the last one is exactly halfway between two bf16 values
+    out = torch.empty(100000, device="cuda", dtype=torch.bfloat16)
+    L.call("sd3_cast_f32_to_bf16", x.data_ptr(), out.data_ptr(), x.numel(), None)
+    assert torch.equal(out, x.bfloat16())

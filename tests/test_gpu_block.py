@@ -1,0 +1,125 @@
+"""One MMDiT-X block on the MI355X against the reference arithmetic: golden vectors of the compiled reference, the CPU
+oracle on the same seeded inputs, a float64 statement of the block at the size of BASELINE config 1, and the bf16 path
+against the fp32 path."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import cases
+import oracle_lib as ol
+from gpu_util import M, dev, dev_params, host, max_abs, rel_l2, F32_TOL, BF16_REL_L2
+from test_oracle import block64
+from sd3_c_amd.params import block_param_shapes, synthetic_params_numpy
+
+pytestmark = pytest.mark.gpu
+GOLDEN = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "reference_outputs.npz"))
+
+
+def run_gpu_block(k, precision="fp32", entry=None):
+    y, c, x = dev(k["y"]), dev(k["c"]), dev(k["x"])
+    B, Tc, Cd = k["c"].shape
+    Tx = k["x"].shape[1]
+    fn = entry or M.Dit_block
+    c_out, x_out = fn(y, c, x, dev_params(k["params"]), B, Tc, Tx, Cd, k["NH"], k["mlp_expand"], k["use_dual"], k["use_qk_norm"], k["discard_context"],
+                      precision=precision)
+    assert c_out.data_ptr() == c.data_ptr() and x_out.data_ptr() == x.data_ptr()  # updated in place, like the reference (modules.cpp:1602)
+    assert np.array_equal(host(y), k["y"])
+    return host(c_out), host(x_out)
+
+
+@pytest.mark.parametrize("name", list(cases.BLOCK_CASES))
+def test_block_fp32_vs_reference_golden_and_oracle(name):
+    k = cases.block_case(name)
+    c, x = run_gpu_block(k)
+    assert max_abs(x, GOLDEN[name + ".x"]) <= F32_TOL
+    co, xo = ol.orc_dit_block(k["y"], k["c"], k["x"], k["params"], k["NH"], k["mlp_expand"], k["use_dual"], k["use_qk_norm"], k["discard_context"])
+    assert max_abs(x, xo) <= F32_TOL
+    if k["discard_context"]:
+        assert np.array_equal(c, k["c"])
+    else:
+        assert max_abs(c, GOLDEN[name + ".c"]) <= F32_TOL and max_abs(c, co) <= F32_TOL
+
+
+def test_block_cuda_entry_point_is_the_same_block():
+    k = cases.block_case("block_dual_hs64")
+    c, x = run_gpu_block(k, entry=M.DiT_block_cuda)
+    assert max_abs(x, GOLDEN["block_dual_hs64.x"]) <= F32_TOL and max_abs(c, GOLDEN["block_dual_hs64.c"]) <= F32_TOL
+
+
+def _wide_case(B, Tc, Tx, dual, discard, seed, C=1536, NH=24, me=4):
+    rng = np.random.Generator(np.random.Philox(seed))
+    params = synthetic_params_numpy(block_param_shapes(C, me, dual, True, discard, C // NH), seed + 1, 0.02, 0.02)
+    return dict(y=rng.standard_normal((B, C), dtype=np.float32), c=rng.standard_normal((B, Tc, C), dtype=np.float32),
+                x=rng.standard_normal((B, Tx, C), dtype=np.float32), params=params, NH=NH, mlp_expand=me, use_dual=dual, use_qk_norm=True,
+                discard_context=discard)
+
+
+@pytest.mark.parametrize("dual,discard", [(True, False), (False, True)])
+def test_block_fp32_width_1536_vs_oracle(dual, discard):
+    """SD3.5-medium width (1536, 24 heads of 64) with few tokens so that the CPU oracle finishes in seconds."""
+    k = _wide_case(2, 5, 19, dual, discard, 11)
+    c, x = run_gpu_block(k)
+    co, xo = ol.orc_dit_block(k["y"], k["c"], k["x"], k["params"], 24, 4, dual, True, discard)
+    assert max_abs(x, xo) <= F32_TOL
+    assert max_abs(c, co) <= F32_TOL
+
+
+@pytest.mark.parametrize("dual", [True, False])
+def test_block_fp32_baseline_config1_vs_float64(dual):
+    """BASELINE config 1 at full size (B=1, 256 image + 77 text tokens, width 1536): the CPU oracle needs a minute for this,
+    so the check is against the float64 numpy statement of the block that tests/test_oracle.py pins to the oracle."""
+    k = _wide_case(1, 77, 256, dual, False, 21)
+    c, x = run_gpu_block(k)
+    c64, x64 = block64(k["y"], k["c"], k["x"], k["params"], 24, dual, True, False)
+    assert max_abs(x, x64) <= F32_TOL and max_abs(c, c64) <= F32_TOL
+
+
+def test_block_zero_gates_is_identity_on_gpu():
+    k = _wide_case(1, 77, 256, True, False, 31)
+    P = dict(k["params"])
+    for pre, nch in (("context_", 6), ("latent_", 9)):
+        w, b = P[pre + "ada_lnorm.linear.weight"].copy(), P[pre + "ada_lnorm.linear.bias"].copy()
+        for g in (2, 5, 8):
+            if g < nch:
+                w[:, g * 1536:(g + 1) * 1536] = 0
+                b[g * 1536:(g + 1) * 1536] = 0
+        P[pre + "ada_lnorm.linear.weight"], P[pre + "ada_lnorm.linear.bias"] = w, b
+    k["params"] = P
+    for prec in ("fp32", "bf16"):
+        c, x = run_gpu_block(k, prec)
+        assert np.array_equal(c, k["c"]) and np.array_equal(x, k["x"])
+
+
+@pytest.mark.parametrize("dual,discard,Tc,Tx", [(True, False, 77, 256), (False, True, 77, 256), (True, False, 154, 1000), (False, False, 0, 130)])
+def test_block_bf16_vs_fp32(dual, discard, Tc, Tx):
+    k = _wide_case(2, Tc, Tx, dual, discard, 41)
+    c32, x32 = run_gpu_block(k, "fp32")
+    c16, x16 = run_gpu_block(k, "bf16")
+    # compare the update the block applied, not the O(1) residual it was added to
+    assert rel_l2(x16 - k["x"], x32 - k["x"]) <= 2 * BF16_REL_L2
+    assert rel_l2(x16, x32) <= BF16_REL_L2
+    if not discard and Tc:
+        assert rel_l2(c16, c32) <= BF16_REL_L2
+
+
+def test_block_missing_weight_and_bad_shapes():
+    from sd3_c_amd import lib as L_
+    k = cases.block_case("block_dual_hs64")
+    P = dict(k["params"])
+    del P["latent_dual_to_qkv.weight"]
+    k2 = dict(k, params=P)
+    with pytest.raises(L_.Sd3Error) as e:
+        run_gpu_block(k2)
+    assert e.value.status == 2  # SD3_ERR_MISSING_PARAM
+    run_gpu_block(dict(k2, use_dual=False, params={n: v for n, v in P.items() if "dual" not in n} | {
+        "latent_ada_lnorm.linear.weight": np.ascontiguousarray(k["params"]["latent_ada_lnorm.linear.weight"][:, :6 * 128]),
+        "latent_ada_lnorm.linear.bias": np.ascontiguousarray(k["params"]["latent_ada_lnorm.linear.bias"][:6 * 128])}))
+    with pytest.raises(L_.Sd3Error) as e:
+        M.Dit_block(dev(k["y"]), dev(k["c"]), dev(k["x"]), dev_params(k["params"]), 1, 7, 16, 128, 3, 4, True, True, False)  # 128 % 3 != 0
+    assert e.value.status == 1
+    with pytest.raises(L_.Sd3Error) as e:
+        run_gpu_block(k, "bf16") if False else M.Dit_block(dev(k["y"]), dev(k["c"]), dev(k["x"]), dev_params(k["params"]), 1, 7, 16, 128, 4, 4, True,
+                                                            True, False, precision="bf16")  # head_dim 32 on the bf16 path
+    assert e.value.status == 3

@@ -1,0 +1,104 @@
+"""Full denoiser forward on the MI355X: fp32 path against golden vectors of the compiled reference and the CPU oracle,
+bf16 path against the fp32 path at the SD3.5-medium shape (BASELINE config 3), and size-independent properties."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import cases
+import oracle_lib as ol
+from gpu_util import M, dev, dev_params, host, max_abs, rel_l2, F32_TOL, BF16_REL_L2
+from sd3_c_amd.config import DiTConfig, sd35_medium
+from sd3_c_amd.params import dit_param_shapes
+
+pytestmark = pytest.mark.gpu
+HERE = os.path.dirname(os.path.abspath(__file__))
+GOLDEN = np.load(os.path.join(HERE, "golden", "reference_outputs.npz"))
+
+
+def run_gpu_dit(k, precision="fp32", params=None):
+    cfg = k["cfg"]
+    args = [dev(k["pooled"]), dev(k["captions"]), dev(k["latent"]), dev(k["timesteps"])]
+    before = [a.clone() for a in args]
+    out = M.DiT(*args, params if params is not None else dev_params(k["params"]), cfg.num_layers, set(cfg.dual_attention_layers), cfg.pooled_dim,
+                cfg.captions_dim, cfg.in_channels, cfg.emb_dim, cfg.attn_heads, cfg.mlp_expand, cfg.patch_size, cfg.pos_embed_max_size, cfg.base_height,
+                cfg.use_qk_norm, precision=precision)
+    for a, b in zip(args, before):
+        assert torch.equal(a, b)  # inputs are left untouched (modules.cpp:1633)
+    return host(out)
+
+
+@pytest.mark.parametrize("name", list(cases.DIT_CASES))
+def test_dit_fp32_vs_reference_golden_and_oracle(name):
+    k = cases.dit_case(name)
+    out = run_gpu_dit(k)
+    assert out.shape == k["latent"].shape
+    assert max_abs(out, GOLDEN[name + ".out"]) <= F32_TOL
+    assert max_abs(out, ol.orc_dit_forward(k["pooled"], k["captions"], k["latent"], k["timesteps"], k["params"], k["cfg"])) <= F32_TOL
+
+
+def test_dit_fp32_reference_test_configuration():
+    """The configuration of the reference's own end-to-end check (module_tests/DiT.py: width 256, 2 heads of 128, 3 blocks,
+    64x64 latent, 154 text tokens), against the output of the compiled reference on the same inputs."""
+    k = cases.dit_reference_test_case()
+    gold = np.load(os.path.join(HERE, "golden", "reference_dit_test_config.npz"))["out"]
+    assert max_abs(run_gpu_dit(k), gold) <= F32_TOL
+
+
+def _synthetic_device_params(cfg, seed):
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    P = {}
+    for name, shape in dit_param_shapes(cfg).items():
+        if "rmsnorm" in name:
+            P[name] = 1 + 0.02 * torch.randn(shape, device="cuda", generator=g)
+        elif name.endswith(".bias"):
+            P[name] = 0.02 * torch.randn(shape, device="cuda", generator=g)
+        else:
+            P[name] = 0.02 * torch.randn(shape, device="cuda", generator=g)
+    return P
+
+
+def _inputs(cfg, B, Tc, H, W, seed):
+    rng = np.random.Generator(np.random.Philox(seed))
+    return dict(cfg=cfg, latent=rng.standard_normal((B, cfg.in_channels, H, W), dtype=np.float32),
+                captions=rng.standard_normal((B, Tc, cfg.captions_dim), dtype=np.float32), pooled=rng.standard_normal((B, cfg.pooled_dim), dtype=np.float32),
+                timesteps=(rng.random((B,), dtype=np.float32) * 1000).astype(np.float32))
+
+
+def test_dit_bf16_vs_fp32_sd35_medium_512px():
+    """BASELINE config 3: full SD3.5-medium shape (24 blocks, width 1536, 13 dual blocks), 64x64 latent = 1024 image tokens,
+    154 text tokens, batch 2. The bf16 path must stay within relative L2 1e-2 of the fp32 path on the final velocity."""
+    cfg = sd35_medium()
+    P = _synthetic_device_params(cfg, 5)
+    k = _inputs(cfg, 2, 154, 64, 64, 6)
+    o32 = run_gpu_dit(k, "fp32", P)
+    o16 = run_gpu_dit(k, "bf16", P)
+    assert np.isfinite(o32).all() and np.isfinite(o16).all()
+    assert rel_l2(o16, o32) <= BF16_REL_L2
+    # batch elements are independent: running element 1 alone gives the same answer (checks batch indexing of every kernel)
+    k1 = dict(k, latent=k["latent"][1:], captions=k["captions"][1:], pooled=k["pooled"][1:], timesteps=k["timesteps"][1:])
+    assert rel_l2(run_gpu_dit(k1, "bf16", P)[0], o16[1]) <= 1e-5
+
+
+def test_dit_ragged_shapes_bf16_vs_fp32():
+    """Token counts that are not multiples of any tile (odd grid, 1 text token), reduced depth."""
+    cfg = DiTConfig(num_layers=3, dual_attention_layers=(0, 1), emb_dim=512, attn_heads=8, pooled_dim=128, captions_dim=192, pos_embed_max_size=64,
+                    base_height=32)
+    P = _synthetic_device_params(cfg, 7)
+    k = _inputs(cfg, 3, 1, 2 * 13, 2 * 9, 8)
+    o32 = run_gpu_dit(k, "fp32", P)
+    assert rel_l2(run_gpu_dit(k, "bf16", P), o32) <= BF16_REL_L2
+    host_P = {n: host(v) for n, v in P.items()}
+    small = dict(k, params=host_P)
+    assert max_abs(o32, ol.orc_dit_forward(k["pooled"], k["captions"], k["latent"], k["timesteps"], host_P, cfg)) <= F32_TOL
+
+
+def test_dit_missing_parameter_is_reported():
+    from sd3_c_amd import lib as L_
+    k = cases.dit_case("dit_small")
+    P = dev_params(k["params"])
+    del P["linear_out.weight"]
+    with pytest.raises(L_.Sd3Error) as e:
+        run_gpu_dit(k, "fp32", P)
+    assert e.value.status == 2 and "linear_out.weight" in str(e.value)
