@@ -1,0 +1,153 @@
+"""Headline benchmark: SD3.5-medium MMDiT-X denoiser forward at 1024x1024 (4096 image + 154 text tokens), batch 2 (a
+classifier-free-guidance pair), bf16 MFMA path, synthetic inputs and random-init weights resident in HBM.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--image 1024] [--no-cpu-baseline]
+
+Prints ONE JSON line. A "step" is one full forward. `roofline` describes the kernel class with the largest share of the
+step time, from HIP events recorded around every launch on the library's stream during the timed steps. `cpu_baseline`
+times the single-threaded CPU oracle on a bounded sample (one block at full width on few tokens) and converts it with
+the FLOP count of a step; it is a reported baseline, not a target."""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
+
+
+def forward_flops(cfg, B, Tc, Tx):
+    """2 FLOP per MAC; attention 4*B*heads*Tq*Tk*head_dim; the last block has no context out-projection / MLP."""
+    C, E = cfg.emb_dim, cfg.mlp_expand
+    gemm = attn = 0.0
+    for l in range(cfg.num_layers):
+        last = l == cfg.num_layers - 1
+        dual = l in cfg.dual_attention_layers
+        per_x = 3 * C * C + C * C + 2 * E * C * C + (4 * C * C if dual else 0)
+        per_c = 3 * C * C + (0 if last else C * C + 2 * E * C * C)
+        gemm += 2.0 * B * (Tx * per_x + Tc * per_c)
+        attn += 4.0 * B * (Tc + Tx) ** 2 * C + (4.0 * B * Tx * Tx * C if dual else 0)
+    p2c = cfg.patch_size ** 2 * cfg.in_channels
+    embed = 2.0 * B * (Tc * cfg.captions_dim * C + Tx * p2c * C + Tx * C * p2c + 256 * C + cfg.pooled_dim * C + 2 * C * C)
+    return gemm, attn, embed
+
+
+def cpu_baseline(cfg, flops_per_step):
+    """Times the CPU oracle (single thread, the reference's loop nests) on ONE dual-attention block at full width on
+    32 image + 8 text tokens, and scales by FLOP to a full step."""
+    import numpy as np
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import oracle_lib as ol
+    from sd3_c_amd.params import block_param_shapes, synthetic_params_numpy
+    B, Tc, Tx, C, NH, E = 1, 8, 32, cfg.emb_dim, cfg.attn_heads, cfg.mlp_expand
+    P = synthetic_params_numpy(block_param_shapes(C, E, True, True, False, C // NH), 3)
+    rng = np.random.Generator(np.random.Philox(4))
+    y, c, x = (rng.standard_normal(s, dtype=np.float32) for s in ((B, C), (B, Tc, C), (B, Tx, C)))
+    t0 = time.perf_counter()
+    ol.orc_dit_block(y, c, x, P, NH, E, True, True, False)
+    dt = time.perf_counter() - t0
+    per_x = 2.0 * (3 + 1 + 2 * E + 4) * C * C
+    per_c = 2.0 * (3 + 1 + 2 * E) * C * C
+    ada = 2.0 * B * 15 * C * C
+    flops = B * (Tx * per_x + Tc * per_c) + ada + 4.0 * B * ((Tc + Tx) ** 2 + Tx * Tx) * C
+    rate = flops / dt
+    return {"value": rate / flops_per_step, "unit": "steps/s", "cores": 1, "kind": "port",
+            "sample": f"oracle/sd3_oracle.c, one dual-attention block at width {C} on {Tx}+{Tc} tokens, batch 1: {flops / 1e9:.2f} GFLOP in {dt:.1f} s "
+                      f"= {rate / 1e9:.3f} GFLOP/s on 1 thread of {os.cpu_count()} visible cores; scaled by FLOP to the {flops_per_step / 1e12:.2f} TFLOP step"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--batch", type=int, default=2)
+    ap.add_argument("--image", type=int, default=1024, help="image side in pixels (latent side = image/8)")
+    ap.add_argument("--precision", default="bf16", choices=["bf16", "fp32"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-events", action="store_true", help="do not record per-kernel events during the timed steps")
+    a = ap.parse_args()
+    if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs on ONE GPU (no collectives, no sharding); use --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from __graft_entry__ import load_package
+    load_package()
+    from sd3_c_amd import modules as M
+    from sd3_c_amd.config import sd35_medium
+    from sd3_c_amd.params import dit_param_shapes
+
+    cfg = sd35_medium()
+    B, Tc, side = a.batch, 154, a.image // 8
+    Tx = cfg.tokens(side, side)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    g = torch.Generator(device=dev).manual_seed(0x5D3 + 4)
+    P = {}
+    for name, shape in dit_param_shapes(cfg).items():
+        if "rmsnorm" in name:
+            P[name] = 1 + 0.02 * torch.randn(shape, device=dev, generator=g)
+        elif name.endswith(".bias"):
+            P[name] = torch.zeros(shape, device=dev)
+        else:
+            P[name] = 0.02 * torch.randn(shape, device=dev, generator=g)
+    latent = torch.randn((B, cfg.in_channels, side, side), device=dev, generator=g)
+    captions = torch.randn((B, Tc, cfg.captions_dim), device=dev, generator=g)
+    pooled = torch.randn((B, cfg.pooled_dim), device=dev, generator=g)
+    timesteps = torch.rand((B,), device=dev, generator=g) * 1000
+    out = torch.empty_like(latent)
+
+    den = M.Denoiser(P, cfg, a.precision)
+    for _ in range(max(a.warmup, 1) if a.warmup else 0):
+        den(pooled, captions, latent, timesteps, out=out)
+    torch.cuda.synchronize()
+    if not a.no_events:
+        den.ctx.profile_begin()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(a.steps):
+        den(pooled, captions, latent, timesteps, out=out)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    prof = den.ctx.profile_end() if not a.no_events else {}
+    assert torch.isfinite(out).all()
+
+    gemm_f, attn_f, embed_f = forward_flops(cfg, B, Tc, Tx)
+    total_f = gemm_f + attn_f + embed_f
+    ms_step = dt / a.steps * 1e3
+    kernels = {}
+    for k, (ms, work, n) in prof.items():
+        if n == 0:
+            continue
+        mfma = k in ("gemm", "attention")
+        ach = work / (ms * 1e-3) / (1e12 if mfma else 1e9)
+        peak = PEAK_BF16_TFLOPS if mfma else PEAK_HBM_GBS
+        kernels[k] = {"bound": "mfma" if mfma else "hbm", "achieved": round(ach, 2), "peak": peak, "unit": "TFLOP/s" if mfma else "GB/s",
+                      "frac": round(ach / peak, 4), "ms_per_step": round(ms / a.steps, 4), "launches_per_step": n // a.steps,
+                      "avg_launch_us": round(ms / n * 1e3, 2)}
+    roofline = None
+    if kernels:
+        dom = max(kernels, key=lambda k: kernels[k]["ms_per_step"])
+        roofline = {"kernel": dom, **{k: kernels[dom][k] for k in ("bound", "achieved", "peak", "unit", "frac")}, "traffic": None}
+    res = {
+        "metric": "DiT fwd steps/s @1024px (4096+154 tok, bf16); GEMM/attn % of MFMA peak",
+        "value": round(a.steps / dt, 3), "unit": "steps/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(ms_step, 3),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": a.precision, "data": "synthetic",
+        "config": {"workload": f"SD3.5-medium MMDiT-X forward, {a.image}x{a.image} image = {Tx} image + {Tc} text tokens, batch {B} (CFG pair), "
+                               f"24 blocks width 1536, 13 dual-attention blocks, random-init weights N(0,0.02)",
+                   "batch": B, "image_tokens": Tx, "text_tokens": Tc, "flop_per_step": total_f},
+        "model_tflops": round(total_f / (dt / a.steps) / 1e12, 2),
+        "roofline": roofline, "kernels": kernels,
+    }
+    if not a.no_cpu_baseline:
+        res["cpu_baseline"] = cpu_baseline(cfg, total_f)
+    print(json.dumps(res))
+
+
+if __name__ == "__main__":
+    main()

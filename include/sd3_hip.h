@@ -19,7 +19,7 @@ extern "C" {
 
 typedef enum sd3_status {
     SD3_OK = 0,
-    SD3_ERR_INVALID_ARG = 1,   /* null pointer, non-positive size, C %% heads != 0 ... */
+    SD3_ERR_INVALID_ARG = 1,   /* null pointer, non-positive size, C % heads != 0 ... */
     SD3_ERR_MISSING_PARAM = 2, /* a weight the requested configuration needs was not bound */
     SD3_ERR_UNSUPPORTED = 3,   /* shape outside what the kernels handle (e.g. head_dim > 128) */
     SD3_ERR_HIP = 4,           /* a HIP runtime call failed; see sd3_last_error() */
@@ -130,6 +130,15 @@ int sd3_dit_forward(sd3_ctx* ctx, const float* pooled, const float* captions, co
                     int emb_dim, int attn_heads, int mlp_expand, int patch_size, int pos_embed_max_size, int base_height, int use_qk_norm,
                     int precision);
 
+/* Per-kernel-class timing (no counterpart in the reference, which has no profiling). Between begin and end every
+ * launch made through `ctx` by sd3_dit_block* / sd3_dit_forward is bracketed by two HIP events on the context's stream.
+ * sd3_profile_end synchronises and returns, per class, the summed event time in ms, the summed algorithmic work
+ * (FLOP for SD3_PROF_GEMM / SD3_PROF_ATTENTION: 2*M*N*K and 4*B*heads*Tq*Tk*head_dim; bytes for the others: each
+ * tensor counted once per read and once per write) and the number of launches. Arrays have SD3_PROF_CLASSES entries. */
+enum { SD3_PROF_GEMM = 0, SD3_PROF_ATTENTION = 1, SD3_PROF_LAYERNORM = 2, SD3_PROF_ADALN = 3, SD3_PROF_CLASSES = 4 };
+int sd3_profile_begin(sd3_ctx* ctx);
+int sd3_profile_end(sd3_ctx* ctx, double* ms, double* work, long long* launches);
+
 /* ------------------------------------------------------------------ bf16 kernels on their own (no counterpart in the reference,
  * whose GPU file is fp32/TF32 only; exposed so that the MFMA kernels can be tested and timed in isolation) */
 
@@ -141,7 +150,7 @@ int sd3_dit_forward(sd3_ctx* ctx, const float* pooled, const float* captions, co
 int sd3_flash_attention_bf16(const void* qkv0, const void* qkv1, void* out0, void* out1, const float* rms_q0, const float* rms_k0,
                              const float* rms_q1, const float* rms_k1, int B, int T0, int T1, int num_heads, int head_dim, void* stream);
 /* out(M,N) = A(M,K) @ W + bias with A bf16 row-major, W given in the reference's fp32 (K,N) layout already packed by
- * sd3_pack_weight_bf16 into `wpacked`; out bf16. K %% 64 == 0 and N %% 8 == 0 required. epilogue: 0 bias, 1 bias+GELU-tanh. */
+ * sd3_pack_weight_bf16 into `wpacked`; out bf16. K % 64 == 0 and N % 8 == 0 required. epilogue: 0 bias, 1 bias+GELU-tanh. */
 int sd3_pack_weight_bf16(const float* W, void* wpacked, int K, int N, void* stream);
 int sd3_gemm_bf16(const void* A, const void* wpacked, const float* bias, void* out, int M, int N, int K, int epilogue, void* stream);
 /* fp32 -> bf16 (round to nearest even) */

@@ -48,6 +48,15 @@ struct sd3_ctx {
     std::map<std::tuple<int, int, int, int, int>, float*> pos_tables;  // (C, max, base, h, w) -> cropped table
     void* ws = nullptr;
     size_t ws_bytes = 0;
+    // optional per-kernel-class timing with HIP events on the context's stream
+    bool prof_on = false;
+    struct ProfSample {
+        hipEvent_t a, b;
+        int cls;
+        double work;
+    };
+    std::vector<ProfSample> prof;
+    std::vector<hipEvent_t> event_pool;
 };
 
 namespace {
@@ -115,6 +124,37 @@ int get_packed(sd3_ctx* ctx, const float* w, long long K, long long N, int kind,
     return SD3_OK;
 }
 
+// Brackets one kernel launch with two events when profiling is on. `work` is the launch's algorithmic work
+// (FLOP for the MFMA classes, bytes for the memory-bound ones).
+struct ProfScope {
+    sd3_ctx* ctx;
+    hipEvent_t a = nullptr, b = nullptr;
+    int cls;
+    double work;
+    ProfScope(sd3_ctx* c, int cls_, double work_) : ctx(c), cls(cls_), work(work_) {
+        if (!ctx->prof_on) return;
+        auto get = [&]() -> hipEvent_t {
+            hipEvent_t e = nullptr;
+            if (!ctx->event_pool.empty()) {
+                e = ctx->event_pool.back();
+                ctx->event_pool.pop_back();
+            } else if (hipEventCreate(&e) != hipSuccess) {
+                (void)hipGetLastError();
+                e = nullptr;
+            }
+            return e;
+        };
+        a = get();
+        b = get();
+        if (a) (void)hipEventRecord(a, ctx->stream);
+    }
+    ~ProfScope() {
+        if (!a || !b) return;
+        (void)hipEventRecord(b, ctx->stream);
+        ctx->prof.push_back({a, b, cls, work});
+    }
+};
+
 struct Dims {
     int B, Tc, Tx, C, NH, HS, E;  // E = mlp_expand
     bool dual, qk, discard;
@@ -138,9 +178,13 @@ int linear_layer(sd3_ctx* ctx, int prec, const void* A, const float* W, const fl
                  GemmEpilogueArgs ea) {
     if (!W) return fail(SD3_ERR_MISSING_PARAM, "a weight needed by this configuration is not bound (N=%d K=%d)", N, K);
     ea.bias = bias;
-    if (prec == SD3_PREC_F32) return gemm_f32((const float*)A, K, W, N, 0, (float*)out, ldc, M, N, K, epi, ea, ctx->stream);
+    if (prec == SD3_PREC_F32) {
+        ProfScope ps(ctx, SD3_PROF_GEMM, 2.0 * M * N * K);
+        return gemm_f32((const float*)A, K, W, N, 0, (float*)out, ldc, M, N, K, epi, ea, ctx->stream);
+    }
     const void* wp = nullptr;
     SD3_TRY(get_packed(ctx, W, K, N, 0, &wp));
+    ProfScope ps(ctx, SD3_PROF_GEMM, 2.0 * M * N * K);
     return gemm_bf16((const bf16_t*)A, (const bf16_t*)wp, out, out_f32, ldc, M, N, K, epi, ea, ctx->stream);
 }
 
@@ -152,7 +196,24 @@ int ada_jobs_run(sd3_ctx* ctx, int prec, const float* y, int B, int C, std::vect
             j.W = wp;
         }
     }
+    double bytes = 0;
+    for (auto& j : jobs) bytes += (double)C * j.N * (prec == SD3_PREC_BF16 ? 2 : 4) + (double)B * j.N * 4;
+    ProfScope ps(ctx, SD3_PROF_ADALN, bytes);
     return small_linear_batched(y, B, C, jobs.data(), (int)jobs.size(), prec == SD3_PREC_BF16, -1, ctx->stream);
+}
+
+// LayerNorm + modulation, timed as a memory-bound launch: reads x once (fp32), writes one or two outputs.
+int ln_mod(sd3_ctx* ctx, const float* x, void* out, void* out2, const float* shift, const float* scale, const float* shift2, const float* scale2,
+           int mod_ld, float eps, int B, int T, int C, int bf) {
+    const double n = (double)B * T * C;
+    ProfScope ps(ctx, SD3_PROF_LAYERNORM, n * 4 + n * (bf ? 2 : 4) * (out2 ? 2 : 1));
+    return layernorm_modulate(x, out, out2, shift, scale, shift2, scale2, mod_ld, eps, B, T, C, bf, ctx->stream);
+}
+
+int attention(sd3_ctx* ctx, const AttnSegments& a, int B, int NH, int HS, bool bf) {
+    const double Tq = a.Tq[0] + a.Tq[1], Tk = a.T[0] + a.T[1];
+    ProfScope ps(ctx, SD3_PROF_ATTENTION, 4.0 * B * NH * Tq * Tk * HS);
+    return bf ? attention_bf16(a, B, NH, HS, ctx->stream) : attention_f32(a, B, NH, HS, ctx->stream);
 }
 
 // The block. ada_c / ada_x: modulation vectors (B, chunks*C) already computed, or null to compute them here.
@@ -205,11 +266,11 @@ int run_block(sd3_ctx* ctx, int prec, const float* y, float* c, float* x, const 
     // ---- context stream up to q,k,v (modules.cpp:1381-1399); with discard_context chunk 0 is the scale, chunk 1 the shift
     const float* c_shift = d.discard ? cchunk(1) : cchunk(0);
     const float* c_scale = d.discard ? cchunk(0) : cchunk(1);
-    SD3_TRY(layernorm_modulate(c, c_hid, nullptr, c_shift, c_scale, nullptr, nullptr, ldc_ada, 1e-6f, B, Tc, C, bf, st));
+    SD3_TRY(ln_mod(ctx, c, c_hid, nullptr, c_shift, c_scale, nullptr, nullptr, ldc_ada, 1e-6f, B, Tc, C, bf));
     SD3_TRY(linear_layer(ctx, prec, c_hid, w.c_qkv_w, w.c_qkv_b, c_qkv, !bf, 3 * C, mc, 3 * C, C, EPI_BIAS, none));
     // ---- latent stream up to q,k,v (modules.cpp:1402-1423); the dual branch's input comes from the same normalised rows
-    SD3_TRY(layernorm_modulate(x, x_hid, d.dual ? x_hid2 : nullptr, xchunk(0), xchunk(1), d.dual ? xchunk(6) : nullptr, d.dual ? xchunk(7) : nullptr,
-                               ldx_ada, 1e-6f, B, Tx, C, bf, st));
+    SD3_TRY(ln_mod(ctx, x, x_hid, d.dual ? x_hid2 : nullptr, xchunk(0), xchunk(1), d.dual ? xchunk(6) : nullptr, d.dual ? xchunk(7) : nullptr, ldx_ada,
+                   1e-6f, B, Tx, C, bf));
     SD3_TRY(linear_layer(ctx, prec, x_hid, w.x_qkv_w, w.x_qkv_b, x_qkv, !bf, 3 * C, mx, 3 * C, C, EPI_BIAS, none));
 
     // ---- joint attention over [context ; latent] (modules.cpp:1427-1432), qk-norm fused (bf16) or done in place first (fp32)
@@ -227,7 +288,7 @@ int run_block(sd3_ctx* ctx, int prec, const float* y, float* c, float* x, const 
         a.ld_qkv[0] = a.ld_qkv[1] = 3 * C; a.ld_out[0] = a.ld_out[1] = C;
         a.T[0] = a.Tq[0] = Tc; a.T[1] = a.Tq[1] = Tx;
         if (d.qk) { a.rms_q[0] = w.c_rms_q; a.rms_k[0] = w.c_rms_k; a.rms_q[1] = w.x_rms_q; a.rms_k[1] = w.x_rms_k; }
-        SD3_TRY(bf ? attention_bf16(a, B, d.NH, d.HS, st) : attention_f32(a, B, d.NH, d.HS, st));
+        SD3_TRY(attention(ctx, a, B, d.NH, d.HS, bf));
     }
     // ---- out-projections with the gate and the residual add in the epilogue (modules.cpp:1435-1436, 1459-1462, 1481-1485)
     GemmEpilogueArgs ge;
@@ -248,20 +309,20 @@ int run_block(sd3_ctx* ctx, int prec, const float* y, float* c, float* x, const 
         a.ld_qkv[0] = a.ld_qkv[1] = 3 * C; a.ld_out[0] = a.ld_out[1] = C;
         a.T[0] = a.Tq[0] = Tx;
         if (d.qk) { a.rms_q[0] = w.x2_rms_q; a.rms_k[0] = w.x2_rms_k; }
-        SD3_TRY(bf ? attention_bf16(a, B, d.NH, d.HS, st) : attention_f32(a, B, d.NH, d.HS, st));
+        SD3_TRY(attention(ctx, a, B, d.NH, d.HS, bf));
         ge.rows_per_batch = Tx; ge.gate = xchunk(8); ge.gate_ld = ldx_ada; ge.resid = x;
         SD3_TRY(linear_layer(ctx, prec, x_att, w.x2_out_w, w.x2_out_b, x, 1, C, mx, C, C, EPI_GATE_RESID, ge));
     }
 
     // ---- context MLP (modules.cpp:1463-1476)
     if (!d.discard) {
-        SD3_TRY(layernorm_modulate(c, c_hid, nullptr, cchunk(3), cchunk(4), nullptr, nullptr, ldc_ada, 1e-6f, B, Tc, C, bf, st));
+        SD3_TRY(ln_mod(ctx, c, c_hid, nullptr, cchunk(3), cchunk(4), nullptr, nullptr, ldc_ada, 1e-6f, B, Tc, C, bf));
         SD3_TRY(linear_layer(ctx, prec, c_hid, w.c_mlp_w1, w.c_mlp_b1, c_mlp, !bf, d.E * C, mc, d.E * C, C, EPI_BIAS_GELU, none));
         ge.rows_per_batch = Tc; ge.gate = cchunk(5); ge.gate_ld = ldc_ada; ge.resid = c;
         SD3_TRY(linear_layer(ctx, prec, c_mlp, w.c_mlp_w2, w.c_mlp_b2, c, 1, C, mc, C, d.E * C, EPI_GATE_RESID, ge));
     }
     // ---- latent MLP (modules.cpp:1488-1504)
-    SD3_TRY(layernorm_modulate(x, x_hid, nullptr, xchunk(3), xchunk(4), nullptr, nullptr, ldx_ada, 1e-6f, B, Tx, C, bf, st));
+    SD3_TRY(ln_mod(ctx, x, x_hid, nullptr, xchunk(3), xchunk(4), nullptr, nullptr, ldx_ada, 1e-6f, B, Tx, C, bf));
     SD3_TRY(linear_layer(ctx, prec, x_hid, w.x_mlp_w1, w.x_mlp_b1, x_mlp, !bf, d.E * C, mx, d.E * C, C, EPI_BIAS_GELU, none));
     ge.rows_per_batch = Tx; ge.gate = xchunk(5); ge.gate_ld = ldx_ada; ge.resid = x;
     SD3_TRY(linear_layer(ctx, prec, x_mlp, w.x_mlp_w2, w.x_mlp_b2, x, 1, C, mx, C, d.E * C, EPI_GATE_RESID, ge));
@@ -516,6 +577,11 @@ int sd3_ctx_destroy(sd3_ctx* ctx) {
         for (auto& kv : ctx->packed) (void)hipFree(kv.second.ptr);
         for (auto& kv : ctx->pos_tables) (void)hipFree(kv.second);
         if (ctx->ws) (void)hipFree(ctx->ws);
+        for (auto& p : ctx->prof) {
+            (void)hipEventDestroy(p.a);
+            (void)hipEventDestroy(p.b);
+        }
+        for (auto e : ctx->event_pool) (void)hipEventDestroy(e);
         (void)hipGetLastError();
     }
     delete ctx;
@@ -547,6 +613,39 @@ int sd3_weights_prepare(sd3_ctx* ctx, int precision) {
     SD3_HIP_TRY(hipStreamSynchronize(ctx->stream));
     for (auto& kv : ctx->packed) (void)hipFree(kv.second.ptr);
     ctx->packed.clear();
+    return SD3_OK;
+}
+
+int sd3_profile_begin(sd3_ctx* ctx) {
+    NOTNULL(ctx);
+    for (auto& p : ctx->prof) {
+        ctx->event_pool.push_back(p.a);
+        ctx->event_pool.push_back(p.b);
+    }
+    ctx->prof.clear();
+    ctx->prof_on = true;
+    return SD3_OK;
+}
+int sd3_profile_end(sd3_ctx* ctx, double* ms, double* work, long long* launches) {
+    NOTNULL(ctx); NOTNULL(ms); NOTNULL(work); NOTNULL(launches);
+    ctx->prof_on = false;
+    DeviceGuard g(ctx->device);
+    SD3_HIP_TRY(hipStreamSynchronize(ctx->stream));
+    for (int i = 0; i < SD3_PROF_CLASSES; i++) {
+        ms[i] = 0;
+        work[i] = 0;
+        launches[i] = 0;
+    }
+    for (auto& p : ctx->prof) {
+        float t = 0.f;
+        SD3_HIP_TRY(hipEventElapsedTime(&t, p.a, p.b));
+        ms[p.cls] += t;
+        work[p.cls] += p.work;
+        launches[p.cls] += 1;
+        ctx->event_pool.push_back(p.a);
+        ctx->event_pool.push_back(p.b);
+    }
+    ctx->prof.clear();
     return SD3_OK;
 }
 
@@ -701,10 +800,12 @@ int sd3_dit_forward(sd3_ctx* ctx, const float* pooled, const float* captions, co
             // the conv weight (C, C_in*p*p) is already (N,K) K-contiguous: its MFMA form is a plain cast
             const void* wp = nullptr;
             SD3_TRY(get_packed(ctx, patch_w, C, Kp, 1, &wp));
+            ProfScope ps(ctx, SD3_PROF_GEMM, 2.0 * B * Tx * C * Kp);
             SD3_TRY(gemm_bf16((const bf16_t*)patches, (const bf16_t*)wp, x, 1, C, B * Tx, C, Kp, EPI_BIAS_ROWADD, ea, st));
         } else {
             const void* wt = nullptr;
             SD3_TRY(get_packed(ctx, patch_w, Kp, C, 2, &wt));
+            ProfScope ps(ctx, SD3_PROF_GEMM, 2.0 * B * Tx * C * Kp);
             SD3_TRY(gemm_f32((const float*)patches, Kp, (const float*)wt, C, 0, x, C, B * Tx, C, Kp, EPI_BIAS_ROWADD, ea, st));
         }
     }
@@ -733,7 +834,7 @@ int sd3_dit_forward(sd3_ctx* ctx, const float* pooled, const float* captions, co
         Bump bws(ctx->ws, ctx->ws_bytes);
         bws.off = block_ws_off;
         void* x_hid = bws.take<char>((size_t)B * Tx * C * (bf ? 2 : 4));
-        SD3_TRY(layernorm_modulate(x, x_hid, nullptr, ada_out + C, ada_out, nullptr, nullptr, 2 * C, 1e-5f, B, Tx, C, bf, st));
+        SD3_TRY(ln_mod(ctx, x, x_hid, nullptr, ada_out + C, ada_out, nullptr, nullptr, 2 * C, 1e-5f, B, Tx, C, bf));
         GemmEpilogueArgs none;
         SD3_TRY(linear_layer(ctx, precision, x_hid, out_w, out_b, tokens, 1, PPC, B * Tx, PPC, C, EPI_BIAS, none));
         SD3_TRY(unpatchify(tokens, out, B, C_in, H, W, p, st));

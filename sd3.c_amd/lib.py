@@ -44,6 +44,8 @@ SIGNATURES = {
     "sd3_weights_prepare": [vp, ci],
     "sd3_dit_block": [vp, vp, vp, vp, cs] + [ci] * 10,
     "sd3_dit_forward": [vp] * 6 + [ci] * 5 + [vp] + [ci] * 12,
+    "sd3_profile_begin": [vp],
+    "sd3_profile_end": [vp, vp, vp, vp],
     "sd3_flash_attention_bf16": [vp] * 8 + [ci] * 5 + [vp],
     "sd3_pack_weight_bf16": [vp, vp, ci, ci, vp],
     "sd3_gemm_bf16": [vp, vp, vp, vp, ci, ci, ci, ci, vp],
@@ -66,6 +68,10 @@ def load():
     if _lib is None:
         if not os.path.exists(LIB_PATH):
             raise FileNotFoundError(f"{LIB_PATH} is missing: build it with `python sd3.c_amd/build.py` (there is no CPU fallback)")
+        # torch ships its own copy of the HIP runtime under the same SONAME (libamdhip64.so.7). Two copies in one process
+        # do not share devices or streams, so torch -- which holds the tensors this library is handed -- is loaded first
+        # and the library then binds to the runtime torch brought in.
+        import torch  # noqa: F401
         lib = C.CDLL(LIB_PATH)
         for name, args in SIGNATURES.items():
             fn = getattr(lib, name)

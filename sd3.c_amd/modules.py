@@ -250,6 +250,18 @@ class Context:
     def synchronize(self):
         L.call("sd3_ctx_synchronize", self._h)
 
+    PROFILE_CLASSES = ("gemm", "attention", "layernorm_modulate", "adaln_linear")
+
+    def profile_begin(self):
+        L.call("sd3_profile_begin", self._h)
+
+    def profile_end(self):
+        """-> {class: (ms, work, launches)}; work is FLOP for gemm/attention and bytes for the memory-bound classes."""
+        n = len(self.PROFILE_CLASSES)
+        ms, work, cnt = (C.c_double * n)(), (C.c_double * n)(), (C.c_longlong * n)()
+        L.call("sd3_profile_end", self._h, C.cast(ms, C.c_void_p), C.cast(work, C.c_void_p), C.cast(cnt, C.c_void_p))
+        return {k: (ms[i], work[i], cnt[i]) for i, k in enumerate(self.PROFILE_CLASSES)}
+
     def close(self):
         if self._h:
             L.load().sd3_ctx_destroy(self._h)
