@@ -201,10 +201,12 @@ __global__ void __launch_bounds__(256) flash_attn_bf16_kernel(SegDev s, float q_
                 psum += p;
             }
         l_run = l_run * alpha + psum;
+        if (__any(alpha != 1.0f)) {  // once the running maxima have settled no lane needs the rescale
 #pragma unroll
-        for (int i = 0; i < 2; i++)
+            for (int i = 0; i < 2; i++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) oacc[i][r] *= alpha;
+                for (int r = 0; r < 16; r++) oacc[i][r] *= alpha;
+        }
 
         // ---- O^T += V^T . P^T ; step j of block kb contracts keys 32kb + 16j + {4lk..4lk+3, 8+4lk..8+4lk+3} ----
 #pragma unroll

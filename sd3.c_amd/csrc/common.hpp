@@ -41,14 +41,18 @@ typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
 
-__device__ __forceinline__ bf16_t f32_to_bf16(float f) {  // round to nearest even; NaN stays NaN
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40);
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return (bf16_t)(u >> 16);
+typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2_t;
+typedef __attribute__((__vector_size__(2 * sizeof(float)))) float f32x2_t;
+// fp32 -> bf16, round to nearest even (the gfx950 v_cvt_pk_bf16_f32 instruction)
+__device__ __forceinline__ bf16_t f32_to_bf16(float f) {
+    const __bf16 r = (__bf16)f;
+    return __builtin_bit_cast(bf16_t, r);
 }
 __device__ __forceinline__ float bf16_to_f32(bf16_t h) { return __uint_as_float(((uint32_t)h) << 16); }
-__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) { return (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16); }
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+    const f32x2_t v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+}
 
 __device__ __forceinline__ float gelu_tanh_f(float x) {
     const float p = 0.7978845608028654f;  // sqrt(2/pi)
