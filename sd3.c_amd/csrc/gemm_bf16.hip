@@ -3,14 +3,19 @@
 //   weight transposed and rounded once by pack_weight_bf16), so that both operands are K-contiguous.
 // It replaces linear / partial_linear of the reference (modules.cpp:475-511) for the QKV, out-projection and MLP
 // layers. Epilogues: bias | bias+GELU-tanh | bias+SiLU | gate*(.)+residual (fp32, in place) | bias + row table.
-// Tile 128x128x64 per workgroup of 4 wavefronts (2x2), each wavefront 64x64 = 2x2 MFMA blocks.
+//
+// Data path: global -> LDS with direct loads (global_load_lds_dwordx4: no registers, no VALU), a ring of STAGES
+// LDS buffers with one workgroup barrier per 64-deep K tile; LDS rows are 128 bytes with the 16-byte chunk index
+// XOR-swizzled by a key of the row, which makes both the linear LDS fill and the 16-byte MFMA operand reads conflict-free.
 #include "common.hpp"
 
 namespace sd3 {
 namespace {
 
-constexpr int BM = 128, BN = 128, BK = 64;
-constexpr int PITCH = BK + 8;  // 144-byte rows: 16 consecutive rows start in 16 different 16-byte bank groups
+constexpr int BK = 64;  // bf16 elements per K tile = 128 bytes per LDS row
+
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+typedef const __attribute__((address_space(1))) void* glb_ptr_t;
 
 struct EpiDev {
     const float* bias;
@@ -21,91 +26,251 @@ struct EpiDev {
     int rows_per_batch;
 };
 
-template <int EPI, bool OUT_F32>
-__global__ void __launch_bounds__(256) gemm_bf16_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ Wp, void* __restrict__ out_, int ldc,
-                                                        int M, int N, int K, EpiDev epi) {
-    __shared__ __attribute__((aligned(16))) bf16_t As[BM * PITCH];
-    __shared__ __attribute__((aligned(16))) bf16_t Bs[BN * PITCH];
+// XOR key of an LDS row: rows r..r+7 get 8 different keys (no conflicts on 8-lane / 32-bank groups) and rows r, r+8 get
+// keys that differ in bit 0 (no conflicts on 16-lane / 64-bank groups either).
+__device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 1); }
+
+// s_waitcnt vmcnt(n) with the other counters left unconstrained (gfx9 encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[15:14])
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+    __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
+}
+
+// Workgroup -> output tile. The hardware hands consecutive workgroup ids to the 8 XCDs in turn, and each XCD has
+// its own L2. Workgroups that land on the same XCD are therefore given a contiguous run of tiles, and runs are walked in
+// bands of GROUP_M tile rows, so that the ~32 tiles an XCD works on at a time share a few A row panels and W column
+// panels inside that L2 instead of each pulling its own panels from the fabric.
+__device__ __forceinline__ void tile_of_workgroup(int tiles_m, int tiles_n, int& tile_m, int& tile_n) {
+    constexpr int XCDS = 8, GROUP_M = 4;
+    const int total = tiles_m * tiles_n, wg = blockIdx.x;
+    const int xcd = wg % XCDS, local = wg / XCDS;
+    const int per = (total + XCDS - 1) / XCDS, tall = (total % XCDS) ? (total % XCDS) : XCDS;  // `tall` XCDs get `per` tiles, the rest per-1
+    const int t = (xcd < tall) ? xcd * per + local : tall * per + (xcd - tall) * (per - 1) + local;
+    const int in_group = GROUP_M * tiles_n, group = t / in_group, first_m = group * GROUP_M;
+    const int gsize = min(tiles_m - first_m, GROUP_M);
+    tile_m = first_m + (t % in_group) % gsize;
+    tile_n = (t % in_group) / gsize;
+}
+
+// LDS bytes of a configuration: the tile ring, or the epilogue staging slabs if those are larger
+template <int BM, int BN, int WM, int WN, int STAGES>
+constexpr int smem_bytes() {
+    constexpr int ring = STAGES * (BM + BN) * 128, epi = WM * WN * 32 * (BN / WN + 4) * 4;
+    return ring > epi ? ring : epi;
+}
+
+template <int BM, int BN, int WM, int WN, int STAGES, int EPI, bool OUT_F32>
+__global__ void __launch_bounds__(WM* WN * 64) gemm_bf16_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ Wp, void* __restrict__ out_,
+                                                                int ldc, int M, int N, int K, EpiDev epi) {
+    constexpr int NT = WM * WN * 64;
+    constexpr int TM = BM / WM / 32, TN = BN / WN / 32;      // 32x32 MFMA blocks per wavefront
+    constexpr int A_BYTES = BM * 128, STAGE_BYTES = (BM + BN) * 128;
+    constexpr int LA = BM * 8 / NT, LB = BN * 8 / NT;        // 16-byte chunks per thread per tile
+    static_assert(BM * 8 % NT == 0 && BN * 8 % NT == 0, "tile rows must divide evenly over the threads");
+    static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0, "wavefront tiles are made of 32x32 blocks");
+    extern __shared__ __attribute__((aligned(1024))) char smem[];
+
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave / WN, wn = wave % WN;
     const int l32 = lane & 31, lk = lane >> 5;
-    const int m_blk = blockIdx.y * BM, n_blk = blockIdx.x * BN;
+    int tile_m, tile_n;
+    tile_of_workgroup((M + BM - 1) / BM, (N + BN - 1) / BN, tile_m, tile_n);
+    const int m_blk = tile_m * BM, n_blk = tile_n * BN;
 
-    // staging: each tile is 128 rows x 128 bytes = 1024 chunks of 16 bytes, 4 per thread; 8 consecutive threads read one row
-    const int ld_row = tid >> 3, ld_kc = (tid & 7) * 8;
-    uint4 ra[4], rb[4];
-    auto load_tiles = [&](int k0) {
+    // ---- loader: chunk q = i*NT + tid lands at LDS byte q*16 of its tile, i.e. row q/8, physical chunk q%8 ----
+    const bf16_t* ga[LA];
+    const bf16_t* gb[LB];
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const int m = m_blk + ld_row + i * 32;
-            ra[i] = (m < M) ? *reinterpret_cast<const uint4*>(A + (long long)m * K + k0 + ld_kc) : make_uint4(0, 0, 0, 0);
-            const int n = n_blk + ld_row + i * 32;
-            rb[i] = (n < N) ? *reinterpret_cast<const uint4*>(Wp + (long long)n * K + k0 + ld_kc) : make_uint4(0, 0, 0, 0);
-        }
-    };
-    auto store_tiles = [&]() {
+    for (int i = 0; i < LA; i++) {
+        const int q = i * NT + tid, row = q >> 3, lc = (q & 7) ^ swz(row);
+        const int m = min(m_blk + row, M - 1);  // rows beyond M re-read the last row; their results are never stored
+        ga[i] = A + (long long)m * K + lc * 8;
+    }
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            *reinterpret_cast<uint4*>(&As[(ld_row + i * 32) * PITCH + ld_kc]) = ra[i];
-            *reinterpret_cast<uint4*>(&Bs[(ld_row + i * 32) * PITCH + ld_kc]) = rb[i];
-        }
+    for (int i = 0; i < LB; i++) {
+        const int q = i * NT + tid, row = q >> 3, lc = (q & 7) ^ swz(row);
+        const int n = min(n_blk + row, N - 1);
+        gb[i] = Wp + (long long)n * K + lc * 8;
+    }
+    auto issue_tile = [&](int kt, int stage) {
+        char* sa = smem + stage * STAGE_BYTES + wave * 1024;
+        char* sb = sa + A_BYTES;
+#pragma unroll
+        for (int i = 0; i < LA; i++) __builtin_amdgcn_global_load_lds((glb_ptr_t)(ga[i] + kt * BK), (lds_ptr_t)(sa + i * NT * 16), 16, 0, 0);
+#pragma unroll
+        for (int i = 0; i < LB; i++) __builtin_amdgcn_global_load_lds((glb_ptr_t)(gb[i] + kt * BK), (lds_ptr_t)(sb + i * NT * 16), 16, 0, 0);
     };
 
-    f32x16_t acc[2][2];
+    f32x16_t acc[TM][TN];
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int i = 0; i < TM; i++)
 #pragma unroll
-        for (int j = 0; j < 2; j++)
+        for (int j = 0; j < TN; j++)
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
-    load_tiles(0);
-    for (int k0 = 0; k0 < K; k0 += BK) {
-        store_tiles();
-        __syncthreads();
-        if (k0 + BK < K) load_tiles(k0 + BK);
+    const int nkt = K / BK;
+#pragma unroll
+    for (int s = 0; s < STAGES - 1; s++)
+        if (s < nkt) issue_tile(s, s);
+
+    // operand addresses inside a stage: row*128 + ((2*ks + lk) ^ sw)*16 with sw = swz(row) = swz(l32) (block offsets are multiples of 16)
+    const int sw = swz(l32);
+    const int a_off = (wm * (BM / WM) + l32) * 128, b_off = A_BYTES + (wn * (BN / WN) + l32) * 128;
+
+    for (int kt = 0; kt < nkt; kt++) {
+        // tile kt has landed once at most (STAGES-2) newer tiles of this thread are still in flight
+        if (kt + STAGES - 1 <= nkt) wait_vmcnt<(STAGES - 2) * (LA + LB)>();
+        else wait_vmcnt<0>();
+        __syncthreads();  // everyone's part of tile kt is in LDS, and everyone is done reading the buffer refilled next
+        if (kt + STAGES - 1 < nkt) issue_tile(kt + STAGES - 1, (kt + STAGES - 1) % STAGES);
+        const char* st = smem + (kt % STAGES) * STAGE_BYTES;
+        // operand fragments of step ks+1 are fetched from LDS while the matrix cores work on step ks
+        bf16x8_t a[2][TM], b[2][TN];
+        auto fetch = [&](int ks, int buf) {
+            const int ch = ((2 * ks + lk) ^ sw) * 16;
+#pragma unroll
+            for (int i = 0; i < TM; i++) a[buf][i] = *reinterpret_cast<const bf16x8_t*>(st + a_off + i * 32 * 128 + ch);
+#pragma unroll
+            for (int j = 0; j < TN; j++) b[buf][j] = *reinterpret_cast<const bf16x8_t*>(st + b_off + j * 32 * 128 + ch);
+        };
+        fetch(0, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, TM + TN, 0);
 #pragma unroll
         for (int ks = 0; ks < BK / 16; ks++) {
-            bf16x8_t a[2], b[2];
+            if (ks + 1 < BK / 16) fetch(ks + 1, (ks + 1) & 1);
 #pragma unroll
-            for (int i = 0; i < 2; i++) a[i] = *reinterpret_cast<const bf16x8_t*>(&As[(wm * 64 + i * 32 + l32) * PITCH + ks * 16 + lk * 8]);
+            for (int i = 0; i < TM; i++)
 #pragma unroll
-            for (int j = 0; j < 2; j++) b[j] = *reinterpret_cast<const bf16x8_t*>(&Bs[(wn * 64 + j * 32 + l32) * PITCH + ks * 16 + lk * 8]);
+                for (int j = 0; j < TN; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[ks & 1][i], b[ks & 1][j], acc[i][j], 0, 0, 0);
+            // scheduling pattern for this step: one LDS fragment read of the next step behind each of the first matrix
+            // instructions, so that LDS latency is covered by matrix work instead of a wait in front of every group
+            if (ks + 1 < BK / 16) {
 #pragma unroll
-            for (int i = 0; i < 2; i++)
-#pragma unroll
-                for (int j = 0; j < 2; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
-        }
-        __syncthreads();
-    }
-
-    // C layout: lane holds column (lane % 32); register r is row 8*(r/4) + 4*(lane/32) + r%4
-    float* outf = reinterpret_cast<float*>(out_);
-    bf16_t* outh = reinterpret_cast<bf16_t*>(out_);
-#pragma unroll
-    for (int i = 0; i < 2; i++)
-#pragma unroll
-        for (int j = 0; j < 2; j++) {
-            const int n = n_blk + wn * 64 + j * 32 + l32;
-            if (n >= N) continue;
-            const float bias = epi.bias ? epi.bias[n] : 0.f;
-#pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const int m = m_blk + wm * 64 + i * 32 + 8 * (r >> 2) + 4 * lk + (r & 3);
-                if (m >= M) continue;
-                const long long idx = (long long)m * ldc + n;
-                float v = acc[i][j][r] + bias;
-                if (EPI == EPI_BIAS_GELU) v = gelu_tanh_f(v);
-                else if (EPI == EPI_BIAS_SILU) v = v / (1.0f + __expf(-v));
-                else if (EPI == EPI_GATE_RESID) v = epi.resid[idx] + epi.gate[(long long)(m / epi.rows_per_batch) * epi.gate_ld + n] * v;
-                else if (EPI == EPI_BIAS_ROWADD) v += epi.table[(long long)(m % epi.rows_per_batch) * epi.gate_ld + n];
-                if (OUT_F32) outf[idx] = v;
-                else outh[idx] = f32_to_bf16(v);
+                for (int x = 0; x < TM + TN; x++) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // 1 DS read
+                }
+                __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - (TM + TN), 0);
+            } else {
+                __builtin_amdgcn_sched_group_barrier(0x008, TM * TN, 0);
             }
         }
+    }
+
+    // ---- epilogue. The MFMA C layout (lane = column, register r = row 8*(r/4) + 4*(lane/32) + r%4) would give 2- or
+    // 4-byte scattered stores; each wavefront instead transposes one 32-row slab at a time through its private LDS
+    // region (the tile ring is free now) and leaves with 16 lanes covering 64 contiguous columns of one row.
+    __syncthreads();
+    constexpr int WNC = BN / WN;        // columns per wavefront
+    constexpr int EP = WNC + 4;         // fp32 pitch of the staging slab
+    static_assert(WM * WN * 32 * EP * 4 <= smem_bytes<BM, BN, WM, WN, STAGES>(), "epilogue staging must fit in the LDS allocation");
+    float* slab = reinterpret_cast<float*>(smem) + wave * 32 * EP;
+    float* outf = reinterpret_cast<float*>(out_);
+    bf16_t* outh = reinterpret_cast<bf16_t*>(out_);
+    constexpr int CPR = WNC / 4;        // float4 chunks per row
+    constexpr int RPI = 64 / CPR;       // rows covered by one pass of the wavefront
+    const int e_row = lane / CPR, e_col = (lane % CPR) * 4;
+    const int n0 = n_blk + wn * WNC + e_col;
+    const bool vec_ok = ((N & 3) == 0) && ((ldc & 3) == 0);
+    const int nvalid = min(4, N - n0);  // <= 0 for lanes beyond the last column
+    float bias4[4] = {0.f, 0.f, 0.f, 0.f};
+    if (epi.bias)
+#pragma unroll
+        for (int c = 0; c < 4; c++)
+            if (c < nvalid) bias4[c] = epi.bias[n0 + c];
+    // batch index of a row without a division per row: the tile starts in batch b0 and crosses a boundary every rpb rows
+    const int rpb = epi.rows_per_batch, b0 = m_blk / rpb;
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) slab[(8 * (r >> 2) + 4 * lk + (r & 3)) * EP + j * 32 + l32] = acc[i][j][r];
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int p = 0; p < 32 / RPI; p++) {
+            const int row = p * RPI + e_row;
+            const int m = m_blk + wm * (BM / WM) + i * 32 + row;
+            if (m < M && nvalid > 0) {
+                const float4 a4 = *reinterpret_cast<const float4*>(&slab[row * EP + e_col]);
+                float v[4] = {a4.x + bias4[0], a4.y + bias4[1], a4.z + bias4[2], a4.w + bias4[3]};
+                const long long idx = (long long)m * ldc + n0;
+                if (EPI == EPI_BIAS_GELU) {
+#pragma unroll
+                    for (int c = 0; c < 4; c++) v[c] = gelu_tanh_f(v[c]);
+                } else if (EPI == EPI_BIAS_SILU) {
+#pragma unroll
+                    for (int c = 0; c < 4; c++) v[c] = v[c] / (1.0f + __expf(-v[c]));
+                } else if (EPI == EPI_GATE_RESID) {
+                    int bi = b0;
+                    for (int nb = (b0 + 1) * rpb; nb <= m; nb += rpb) bi++;  // at most BM/rpb + 1 steps, 0 or 1 in practice
+                    const float* g = epi.gate + (long long)bi * epi.gate_ld + n0;
+                    if (vec_ok) {
+                        const float4 g4 = *reinterpret_cast<const float4*>(g), r4 = *reinterpret_cast<const float4*>(epi.resid + idx);
+                        v[0] = r4.x + g4.x * v[0]; v[1] = r4.y + g4.y * v[1]; v[2] = r4.z + g4.z * v[2]; v[3] = r4.w + g4.w * v[3];
+                    } else {
+#pragma unroll
+                        for (int c = 0; c < 4; c++)
+                            if (c < nvalid) v[c] = epi.resid[idx + c] + g[c] * v[c];
+                    }
+                } else if (EPI == EPI_BIAS_ROWADD) {
+                    const float* t = epi.table + (long long)(m % rpb) * epi.gate_ld + n0;
+#pragma unroll
+                    for (int c = 0; c < 4; c++)
+                        if (c < nvalid) v[c] += t[c];
+                }
+                if (vec_ok) {
+                    if (OUT_F32) *reinterpret_cast<float4*>(outf + idx) = make_float4(v[0], v[1], v[2], v[3]);
+                    else *reinterpret_cast<uint2*>(outh + idx) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+                } else {
+#pragma unroll
+                    for (int c = 0; c < 4; c++)
+                        if (c < nvalid) {
+                            if (OUT_F32) outf[idx + c] = v[c];
+                            else outh[idx + c] = f32_to_bf16(v[c]);
+                        }
+                }
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+    }
+}
+
+template <int BM, int BN, int WM, int WN, int STAGES, int EPI, bool OUT_F32>
+int launch_cfg(const bf16_t* A, const bf16_t* Wp, void* out, int ldc, int M, int N, int K, const EpiDev& e, hipStream_t st) {
+    auto kern = gemm_bf16_kernel<BM, BN, WM, WN, STAGES, EPI, OUT_F32>;
+    constexpr int smem = smem_bytes<BM, BN, WM, WN, STAGES>();
+    static bool attr_done = false;  // raising the dynamic LDS limit is a per-function, per-process setting
+    if (smem > 65536 && !attr_done) {
+        SD3_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem));
+        attr_done = true;
+    }
+    dim3 grid(((N + BN - 1) / BN) * ((M + BM - 1) / BM)), block(WM * WN * 64);
+    hipLaunchKernelGGL(kern, grid, block, smem, st, A, Wp, out, ldc, M, N, K, e);
+    return launch_status("gemm_bf16");
+}
+
+template <int EPI, bool OUT_F32>
+int launch_epi(int variant, const bf16_t* A, const bf16_t* Wp, void* out, int ldc, int M, int N, int K, const EpiDev& e, hipStream_t st) {
+    switch (variant) {
+        case 1: return launch_cfg<128, 256, 2, 2, 2, EPI, OUT_F32>(A, Wp, out, ldc, M, N, K, e, st);
+        case 2: return launch_cfg<256, 128, 2, 2, 2, EPI, OUT_F32>(A, Wp, out, ldc, M, N, K, e, st);
+        case 3: return launch_cfg<256, 128, 2, 2, 3, EPI, OUT_F32>(A, Wp, out, ldc, M, N, K, e, st);
+        case 4: return launch_cfg<256, 256, 2, 4, 2, EPI, OUT_F32>(A, Wp, out, ldc, M, N, K, e, st);
+        case 5: return launch_cfg<256, 256, 4, 2, 2, EPI, OUT_F32>(A, Wp, out, ldc, M, N, K, e, st);
+        case 6: return launch_cfg<128, 128, 2, 2, 3, EPI, OUT_F32>(A, Wp, out, ldc, M, N, K, e, st);
+        default: return launch_cfg<128, 128, 2, 2, 2, EPI, OUT_F32>(A, Wp, out, ldc, M, N, K, e, st);
+    }
 }
 
 }  // namespace
+
+int g_gemm_bf16_variant = -1;  // -1: choose by shape; >= 0: tuning knob (tile shape / pipeline depth), see launch_epi
 
 int gemm_bf16(const bf16_t* A, const bf16_t* Wp, void* out, int out_is_f32, int ldc, int M, int N, int K, int epi, const GemmEpilogueArgs& ea,
               hipStream_t st) {
@@ -115,22 +280,24 @@ int gemm_bf16(const bf16_t* A, const bf16_t* Wp, void* out, int out_is_f32, int 
         return fail(SD3_ERR_INVALID_ARG, "gemm_bf16: operands must be 16-byte aligned");
     EpiDev e{ea.bias, ea.gate, ea.resid, ea.table, ea.gate_ld, ea.rows_per_batch > 0 ? ea.rows_per_batch : 1};
     if (epi == EPI_BIAS_ROWADD) e.gate_ld = N;
-    dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM), block(256);
-#define SD3_GEMM_BF16_LAUNCH(E)                                                                                                \
-    do {                                                                                                                       \
-        if (out_is_f32) hipLaunchKernelGGL((gemm_bf16_kernel<E, true>), grid, block, 0, st, A, Wp, out, ldc, M, N, K, e);      \
-        else hipLaunchKernelGGL((gemm_bf16_kernel<E, false>), grid, block, 0, st, A, Wp, out, ldc, M, N, K, e);                \
-    } while (0)
+    // tile shape: 256x256 (8 wavefronts) for large problems, 128x128 (4 wavefronts) when there are few rows
+    const int v = g_gemm_bf16_variant >= 0 ? g_gemm_bf16_variant : (M >= 1024 ? 4 : 0);
+#define SD3_GEMM_BF16_LAUNCH(E) \
+    return out_is_f32 ? launch_epi<E, true>(v, A, Wp, out, ldc, M, N, K, e, st) : launch_epi<E, false>(v, A, Wp, out, ldc, M, N, K, e, st)
     switch (epi) {
-        case EPI_BIAS: SD3_GEMM_BF16_LAUNCH(EPI_BIAS); break;
-        case EPI_BIAS_GELU: SD3_GEMM_BF16_LAUNCH(EPI_BIAS_GELU); break;
-        case EPI_BIAS_SILU: SD3_GEMM_BF16_LAUNCH(EPI_BIAS_SILU); break;
-        case EPI_GATE_RESID: SD3_GEMM_BF16_LAUNCH(EPI_GATE_RESID); break;
-        case EPI_BIAS_ROWADD: SD3_GEMM_BF16_LAUNCH(EPI_BIAS_ROWADD); break;
+        case EPI_BIAS: SD3_GEMM_BF16_LAUNCH(EPI_BIAS);
+        case EPI_BIAS_GELU: SD3_GEMM_BF16_LAUNCH(EPI_BIAS_GELU);
+        case EPI_BIAS_SILU: SD3_GEMM_BF16_LAUNCH(EPI_BIAS_SILU);
+        case EPI_GATE_RESID: SD3_GEMM_BF16_LAUNCH(EPI_GATE_RESID);
+        case EPI_BIAS_ROWADD: SD3_GEMM_BF16_LAUNCH(EPI_BIAS_ROWADD);
         default: return fail(SD3_ERR_INVALID_ARG, "gemm_bf16: unknown epilogue %d", epi);
     }
 #undef SD3_GEMM_BF16_LAUNCH
-    return launch_status("gemm_bf16");
 }
 
 }  // namespace sd3
+
+extern "C" int sd3_dev_set_gemm_variant(int v) {
+    sd3::g_gemm_bf16_variant = v;
+    return 0;
+}
