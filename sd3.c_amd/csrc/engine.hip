@@ -188,6 +188,43 @@ int linear_layer(sd3_ctx* ctx, int prec, const void* A, const float* W, const fl
     return gemm_bf16((const bf16_t*)A, (const bf16_t*)wp, out, out_f32, ldc, M, N, K, epi, ea, ctx->stream);
 }
 
+// The same layer of the latent stream and of the context stream (different weights and rows, same kind): on the bf16
+// path both go into one launch, so that the few context rows ride along instead of paying a launch of their own.
+struct LayerCall {
+    const void* A;
+    const float* W;
+    const float* bias;
+    void* out;
+    int ldc, M, N, K;
+    GemmEpilogueArgs ea;
+};
+int linear_pair(sd3_ctx* ctx, int prec, const LayerCall* calls, int n, int out_f32, int epi) {
+    if (prec == SD3_PREC_F32) {
+        for (int i = 0; i < n; i++) {
+            const LayerCall& c = calls[i];
+            if (c.M > 0) SD3_TRY(linear_layer(ctx, prec, c.A, c.W, c.bias, c.out, out_f32, c.ldc, c.M, c.N, c.K, epi, c.ea));
+        }
+        return SD3_OK;
+    }
+    GemmBf16Problem probs[2];
+    int m = 0;
+    double flop = 0;
+    for (int i = 0; i < n; i++) {
+        const LayerCall& c = calls[i];
+        if (c.M <= 0) continue;
+        if (!c.W) return fail(SD3_ERR_MISSING_PARAM, "a weight needed by this configuration is not bound (N=%d K=%d)", c.N, c.K);
+        const void* wp = nullptr;
+        SD3_TRY(get_packed(ctx, c.W, c.K, c.N, 0, &wp));
+        probs[m] = GemmBf16Problem{(const bf16_t*)c.A, (const bf16_t*)wp, c.out, c.ldc, c.M, c.N, c.K, c.ea};
+        probs[m].ea.bias = c.bias;
+        flop += 2.0 * c.M * c.N * c.K;
+        m++;
+    }
+    if (m == 0) return SD3_OK;
+    ProfScope ps(ctx, SD3_PROF_GEMM, flop);
+    return gemm_bf16_grouped(probs, m, out_f32, epi, ctx->stream);
+}
+
 int ada_jobs_run(sd3_ctx* ctx, int prec, const float* y, int B, int C, std::vector<SmallLinearJob>& jobs) {
     if (prec == SD3_PREC_BF16) {
         for (auto& j : jobs) {
@@ -263,15 +300,17 @@ int run_block(sd3_ctx* ctx, int prec, const float* y, float* c, float* x, const 
     auto xchunk = [&](int k) { return ada_x + (size_t)k * C; };
     GemmEpilogueArgs none;
 
-    // ---- context stream up to q,k,v (modules.cpp:1381-1399); with discard_context chunk 0 is the scale, chunk 1 the shift
+    // ---- both streams up to q,k,v (modules.cpp:1381-1423); with discard_context chunk 0 is the scale, chunk 1 the shift;
+    //      the dual branch's input comes from the same normalised latent rows
     const float* c_shift = d.discard ? cchunk(1) : cchunk(0);
     const float* c_scale = d.discard ? cchunk(0) : cchunk(1);
-    SD3_TRY(ln_mod(ctx, c, c_hid, nullptr, c_shift, c_scale, nullptr, nullptr, ldc_ada, 1e-6f, B, Tc, C, bf));
-    SD3_TRY(linear_layer(ctx, prec, c_hid, w.c_qkv_w, w.c_qkv_b, c_qkv, !bf, 3 * C, mc, 3 * C, C, EPI_BIAS, none));
-    // ---- latent stream up to q,k,v (modules.cpp:1402-1423); the dual branch's input comes from the same normalised rows
+    if (mc > 0) SD3_TRY(ln_mod(ctx, c, c_hid, nullptr, c_shift, c_scale, nullptr, nullptr, ldc_ada, 1e-6f, B, Tc, C, bf));
     SD3_TRY(ln_mod(ctx, x, x_hid, d.dual ? x_hid2 : nullptr, xchunk(0), xchunk(1), d.dual ? xchunk(6) : nullptr, d.dual ? xchunk(7) : nullptr, ldx_ada,
                    1e-6f, B, Tx, C, bf));
-    SD3_TRY(linear_layer(ctx, prec, x_hid, w.x_qkv_w, w.x_qkv_b, x_qkv, !bf, 3 * C, mx, 3 * C, C, EPI_BIAS, none));
+    {
+        LayerCall qkv[2] = {{x_hid, w.x_qkv_w, w.x_qkv_b, x_qkv, 3 * C, mx, 3 * C, C, none}, {c_hid, w.c_qkv_w, w.c_qkv_b, c_qkv, 3 * C, mc, 3 * C, C, none}};
+        SD3_TRY(linear_pair(ctx, prec, qkv, 2, !bf, EPI_BIAS));
+    }
 
     // ---- joint attention over [context ; latent] (modules.cpp:1427-1432), qk-norm fused (bf16) or done in place first (fp32)
     auto seg_ptr = [&](void* base, int third) -> void* { return (char*)base + (size_t)third * C * es; };
@@ -291,11 +330,13 @@ int run_block(sd3_ctx* ctx, int prec, const float* y, float* c, float* x, const 
         SD3_TRY(attention(ctx, a, B, d.NH, d.HS, bf));
     }
     // ---- out-projections with the gate and the residual add in the epilogue (modules.cpp:1435-1436, 1459-1462, 1481-1485)
-    GemmEpilogueArgs ge;
-    ge.rows_per_batch = Tc; ge.gate = cchunk(2); ge.gate_ld = ldc_ada; ge.resid = c;
-    if (!d.discard) SD3_TRY(linear_layer(ctx, prec, c_att, w.c_out_w, w.c_out_b, c, 1, C, mc, C, C, EPI_GATE_RESID, ge));
-    ge.rows_per_batch = Tx; ge.gate = xchunk(2); ge.gate_ld = ldx_ada; ge.resid = x;
-    SD3_TRY(linear_layer(ctx, prec, x_att, w.x_out_w, w.x_out_b, x, 1, C, mx, C, C, EPI_GATE_RESID, ge));
+    GemmEpilogueArgs gx, gc;
+    gc.rows_per_batch = Tc; gc.gate = cchunk(2); gc.gate_ld = ldc_ada; gc.resid = c;
+    gx.rows_per_batch = Tx; gx.gate = xchunk(2); gx.gate_ld = ldx_ada; gx.resid = x;
+    {
+        LayerCall proj[2] = {{x_att, w.x_out_w, w.x_out_b, x, C, mx, C, C, gx}, {c_att, w.c_out_w, w.c_out_b, c, C, d.discard ? 0 : mc, C, C, gc}};
+        SD3_TRY(linear_pair(ctx, prec, proj, 2, 1, EPI_GATE_RESID));
+    }
 
     // ---- extra self-attention over the latent tokens (modules.cpp:1440-1453, 1486)
     if (d.dual) {
@@ -310,22 +351,24 @@ int run_block(sd3_ctx* ctx, int prec, const float* y, float* c, float* x, const 
         a.T[0] = a.Tq[0] = Tx;
         if (d.qk) { a.rms_q[0] = w.x2_rms_q; a.rms_k[0] = w.x2_rms_k; }
         SD3_TRY(attention(ctx, a, B, d.NH, d.HS, bf));
-        ge.rows_per_batch = Tx; ge.gate = xchunk(8); ge.gate_ld = ldx_ada; ge.resid = x;
-        SD3_TRY(linear_layer(ctx, prec, x_att, w.x2_out_w, w.x2_out_b, x, 1, C, mx, C, C, EPI_GATE_RESID, ge));
+        GemmEpilogueArgs g2;
+        g2.rows_per_batch = Tx; g2.gate = xchunk(8); g2.gate_ld = ldx_ada; g2.resid = x;
+        SD3_TRY(linear_layer(ctx, prec, x_att, w.x2_out_w, w.x2_out_b, x, 1, C, mx, C, C, EPI_GATE_RESID, g2));
     }
 
-    // ---- context MLP (modules.cpp:1463-1476)
-    if (!d.discard) {
-        SD3_TRY(ln_mod(ctx, c, c_hid, nullptr, cchunk(3), cchunk(4), nullptr, nullptr, ldc_ada, 1e-6f, B, Tc, C, bf));
-        SD3_TRY(linear_layer(ctx, prec, c_hid, w.c_mlp_w1, w.c_mlp_b1, c_mlp, !bf, d.E * C, mc, d.E * C, C, EPI_BIAS_GELU, none));
-        ge.rows_per_batch = Tc; ge.gate = cchunk(5); ge.gate_ld = ldc_ada; ge.resid = c;
-        SD3_TRY(linear_layer(ctx, prec, c_mlp, w.c_mlp_w2, w.c_mlp_b2, c, 1, C, mc, C, d.E * C, EPI_GATE_RESID, ge));
-    }
-    // ---- latent MLP (modules.cpp:1488-1504)
+    // ---- MLPs of both streams (modules.cpp:1463-1476, 1488-1504)
+    const int mcm = d.discard ? 0 : mc;
+    if (mcm > 0) SD3_TRY(ln_mod(ctx, c, c_hid, nullptr, cchunk(3), cchunk(4), nullptr, nullptr, ldc_ada, 1e-6f, B, Tc, C, bf));
     SD3_TRY(ln_mod(ctx, x, x_hid, nullptr, xchunk(3), xchunk(4), nullptr, nullptr, ldx_ada, 1e-6f, B, Tx, C, bf));
-    SD3_TRY(linear_layer(ctx, prec, x_hid, w.x_mlp_w1, w.x_mlp_b1, x_mlp, !bf, d.E * C, mx, d.E * C, C, EPI_BIAS_GELU, none));
-    ge.rows_per_batch = Tx; ge.gate = xchunk(5); ge.gate_ld = ldx_ada; ge.resid = x;
-    SD3_TRY(linear_layer(ctx, prec, x_mlp, w.x_mlp_w2, w.x_mlp_b2, x, 1, C, mx, C, d.E * C, EPI_GATE_RESID, ge));
+    {
+        LayerCall up[2] = {{x_hid, w.x_mlp_w1, w.x_mlp_b1, x_mlp, d.E * C, mx, d.E * C, C, none},
+                           {c_hid, w.c_mlp_w1, w.c_mlp_b1, c_mlp, d.E * C, mcm, d.E * C, C, none}};
+        SD3_TRY(linear_pair(ctx, prec, up, 2, !bf, EPI_BIAS_GELU));
+        gc.gate = cchunk(5);
+        gx.gate = xchunk(5);
+        LayerCall down[2] = {{x_mlp, w.x_mlp_w2, w.x_mlp_b2, x, C, mx, C, d.E * C, gx}, {c_mlp, w.c_mlp_w2, w.c_mlp_b2, c, C, mcm, C, d.E * C, gc}};
+        SD3_TRY(linear_pair(ctx, prec, down, 2, 1, EPI_GATE_RESID));
+    }
     return SD3_OK;
 }
 

@@ -41,9 +41,9 @@ __device__ __forceinline__ void wait_vmcnt() {
 // its own L2. Workgroups that land on the same XCD are therefore given a contiguous run of tiles, and runs are walked in
 // bands of GROUP_M tile rows, so that the ~32 tiles an XCD works on at a time share a few A row panels and W column
 // panels inside that L2 instead of each pulling its own panels from the fabric.
-__device__ __forceinline__ void tile_of_workgroup(int tiles_m, int tiles_n, int& tile_m, int& tile_n) {
+__device__ __forceinline__ void tile_of_workgroup(int wg, int tiles_m, int tiles_n, int& tile_m, int& tile_n) {
     constexpr int XCDS = 8, GROUP_M = 4;
-    const int total = tiles_m * tiles_n, wg = blockIdx.x;
+    const int total = tiles_m * tiles_n;
     const int xcd = wg % XCDS, local = wg / XCDS;
     const int per = (total + XCDS - 1) / XCDS, tall = (total % XCDS) ? (total % XCDS) : XCDS;  // `tall` XCDs get `per` tiles, the rest per-1
     const int t = (xcd < tall) ? xcd * per + local : tall * per + (xcd - tall) * (per - 1) + local;
@@ -60,9 +60,30 @@ constexpr int smem_bytes() {
     return ring > epi ? ring : epi;
 }
 
+// One launch covers up to two independent problems (the latent-stream and the context-stream layer of the same kind):
+// workgroups [0, tiles0) belong to problem 0, the rest to problem 1.
+struct Prob {
+    const bf16_t* A;
+    const bf16_t* Wp;
+    void* out;
+    int ldc, M, N, K;
+    EpiDev epi;
+};
+struct ProbPair {
+    Prob p[2];
+    int tiles0;
+};
+
 template <int BM, int BN, int WM, int WN, int STAGES, int EPI, bool OUT_F32>
-__global__ void __launch_bounds__(WM* WN * 64) gemm_bf16_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ Wp, void* __restrict__ out_,
-                                                                int ldc, int M, int N, int K, EpiDev epi) {
+__global__ void __launch_bounds__(WM* WN * 64) gemm_bf16_kernel(const ProbPair args) {
+    const int which = (int)blockIdx.x >= args.tiles0 ? 1 : 0;
+    const int wg = (int)blockIdx.x - (which ? args.tiles0 : 0);
+    const Prob& pr = args.p[which];
+    const bf16_t* __restrict__ A = pr.A;
+    const bf16_t* __restrict__ Wp = pr.Wp;
+    void* __restrict__ out_ = pr.out;
+    const int ldc = pr.ldc, M = pr.M, N = pr.N, K = pr.K;
+    const EpiDev epi = pr.epi;
     constexpr int NT = WM * WN * 64;
     constexpr int TM = BM / WM / 32, TN = BN / WN / 32;      // 32x32 MFMA blocks per wavefront
     constexpr int A_BYTES = BM * 128, STAGE_BYTES = (BM + BN) * 128;
@@ -75,7 +96,7 @@ __global__ void __launch_bounds__(WM* WN * 64) gemm_bf16_kernel(const bf16_t* __
     const int wm = wave / WN, wn = wave % WN;
     const int l32 = lane & 31, lk = lane >> 5;
     int tile_m, tile_n;
-    tile_of_workgroup((M + BM - 1) / BM, (N + BN - 1) / BN, tile_m, tile_n);
+    tile_of_workgroup(wg, (M + BM - 1) / BM, (N + BN - 1) / BN, tile_m, tile_n);
     const int m_blk = tile_m * BM, n_blk = tile_n * BN;
 
     // ---- loader: chunk q = i*NT + tid lands at LDS byte q*16 of its tile, i.e. row q/8, physical chunk q%8 ----
@@ -242,7 +263,7 @@ __global__ void __launch_bounds__(WM* WN * 64) gemm_bf16_kernel(const bf16_t* __
 }
 
 template <int BM, int BN, int WM, int WN, int STAGES, int EPI, bool OUT_F32>
-int launch_cfg(const bf16_t* A, const bf16_t* Wp, void* out, int ldc, int M, int N, int K, const EpiDev& e, hipStream_t st) {
+int launch_cfg(ProbPair& args, int n, hipStream_t st) {
     auto kern = gemm_bf16_kernel<BM, BN, WM, WN, STAGES, EPI, OUT_F32>;
     constexpr int smem = smem_bytes<BM, BN, WM, WN, STAGES>();
     static bool attr_done = false;  // raising the dynamic LDS limit is a per-function, per-process setting
@@ -250,40 +271,48 @@ int launch_cfg(const bf16_t* A, const bf16_t* Wp, void* out, int ldc, int M, int
         SD3_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem));
         attr_done = true;
     }
-    dim3 grid(((N + BN - 1) / BN) * ((M + BM - 1) / BM)), block(WM * WN * 64);
-    hipLaunchKernelGGL(kern, grid, block, smem, st, A, Wp, out, ldc, M, N, K, e);
+    int tiles[2] = {0, 0};
+    for (int i = 0; i < n; i++) tiles[i] = ((args.p[i].N + BN - 1) / BN) * ((args.p[i].M + BM - 1) / BM);
+    args.tiles0 = tiles[0];
+    dim3 grid(tiles[0] + tiles[1]), block(WM * WN * 64);
+    hipLaunchKernelGGL(kern, grid, block, smem, st, args);
     return launch_status("gemm_bf16");
 }
 
 template <int EPI, bool OUT_F32>
-int launch_epi(int variant, const bf16_t* A, const bf16_t* Wp, void* out, int ldc, int M, int N, int K, const EpiDev& e, hipStream_t st) {
+int launch_epi(int variant, ProbPair& args, int n, hipStream_t st) {
     switch (variant) {
-        case 1: return launch_cfg<128, 256, 2, 2, 2, EPI, OUT_F32>(A, Wp, out, ldc, M, N, K, e, st);
-        case 2: return launch_cfg<256, 128, 2, 2, 2, EPI, OUT_F32>(A, Wp, out, ldc, M, N, K, e, st);
-        case 3: return launch_cfg<256, 128, 2, 2, 3, EPI, OUT_F32>(A, Wp, out, ldc, M, N, K, e, st);
-        case 4: return launch_cfg<256, 256, 2, 4, 2, EPI, OUT_F32>(A, Wp, out, ldc, M, N, K, e, st);
-        case 5: return launch_cfg<256, 256, 4, 2, 2, EPI, OUT_F32>(A, Wp, out, ldc, M, N, K, e, st);
-        case 6: return launch_cfg<128, 128, 2, 2, 3, EPI, OUT_F32>(A, Wp, out, ldc, M, N, K, e, st);
-        default: return launch_cfg<128, 128, 2, 2, 2, EPI, OUT_F32>(A, Wp, out, ldc, M, N, K, e, st);
+        case 1: return launch_cfg<128, 256, 2, 2, 2, EPI, OUT_F32>(args, n, st);
+        case 2: return launch_cfg<256, 128, 2, 2, 2, EPI, OUT_F32>(args, n, st);
+        case 4: return launch_cfg<256, 256, 2, 4, 2, EPI, OUT_F32>(args, n, st);
+        default: return launch_cfg<128, 128, 2, 2, 2, EPI, OUT_F32>(args, n, st);
     }
 }
 
 }  // namespace
 
-int g_gemm_bf16_variant = -1;  // -1: choose by shape; >= 0: tuning knob (tile shape / pipeline depth), see launch_epi
+int g_gemm_bf16_variant = -1;  // -1: choose by shape; >= 0: tuning knob (tile shape), see launch_epi
 
-int gemm_bf16(const bf16_t* A, const bf16_t* Wp, void* out, int out_is_f32, int ldc, int M, int N, int K, int epi, const GemmEpilogueArgs& ea,
-              hipStream_t st) {
-    if (M <= 0 || N <= 0) return SD3_OK;
-    if (K <= 0 || (K % BK) != 0) return fail(SD3_ERR_UNSUPPORTED, "gemm_bf16: K=%d must be a positive multiple of %d", K, BK);
-    if ((reinterpret_cast<uintptr_t>(A) & 15) || (reinterpret_cast<uintptr_t>(Wp) & 15))
-        return fail(SD3_ERR_INVALID_ARG, "gemm_bf16: operands must be 16-byte aligned");
-    EpiDev e{ea.bias, ea.gate, ea.resid, ea.table, ea.gate_ld, ea.rows_per_batch > 0 ? ea.rows_per_batch : 1};
-    if (epi == EPI_BIAS_ROWADD) e.gate_ld = N;
+int gemm_bf16_grouped(const GemmBf16Problem* probs, int n, int out_is_f32, int epi, hipStream_t st) {
+    if (n < 1 || n > 2) return fail(SD3_ERR_INVALID_ARG, "gemm_bf16_grouped: 1 or 2 problems (got %d)", n);
+    ProbPair args{};
+    int m = 0, max_M = 0;
+    for (int i = 0; i < n; i++) {
+        const GemmBf16Problem& q = probs[i];
+        if (q.M <= 0 || q.N <= 0) continue;  // an empty problem simply contributes no tiles
+        if (q.K <= 0 || (q.K % BK) != 0) return fail(SD3_ERR_UNSUPPORTED, "gemm_bf16: K=%d must be a positive multiple of %d", q.K, BK);
+        if ((reinterpret_cast<uintptr_t>(q.A) & 15) || (reinterpret_cast<uintptr_t>(q.Wp) & 15))
+            return fail(SD3_ERR_INVALID_ARG, "gemm_bf16: operands must be 16-byte aligned");
+        Prob& d = args.p[m++];
+        d.A = q.A; d.Wp = q.Wp; d.out = q.out; d.ldc = q.ldc; d.M = q.M; d.N = q.N; d.K = q.K;
+        d.epi = EpiDev{q.ea.bias, q.ea.gate, q.ea.resid, q.ea.table, q.ea.gate_ld, q.ea.rows_per_batch > 0 ? q.ea.rows_per_batch : 1};
+        if (epi == EPI_BIAS_ROWADD) d.epi.gate_ld = q.N;
+        if (q.M > max_M) max_M = q.M;
+    }
+    if (m == 0) return SD3_OK;
     // tile shape: 256x256 (8 wavefronts) for large problems, 128x128 (4 wavefronts) when there are few rows
-    const int v = g_gemm_bf16_variant >= 0 ? g_gemm_bf16_variant : (M >= 1024 ? 4 : 0);
-#define SD3_GEMM_BF16_LAUNCH(E) \
-    return out_is_f32 ? launch_epi<E, true>(v, A, Wp, out, ldc, M, N, K, e, st) : launch_epi<E, false>(v, A, Wp, out, ldc, M, N, K, e, st)
+    const int v = g_gemm_bf16_variant >= 0 ? g_gemm_bf16_variant : (max_M >= 1024 ? 4 : 0);
+#define SD3_GEMM_BF16_LAUNCH(E) return out_is_f32 ? launch_epi<E, true>(v, args, m, st) : launch_epi<E, false>(v, args, m, st)
     switch (epi) {
         case EPI_BIAS: SD3_GEMM_BF16_LAUNCH(EPI_BIAS);
         case EPI_BIAS_GELU: SD3_GEMM_BF16_LAUNCH(EPI_BIAS_GELU);
@@ -293,6 +322,12 @@ int gemm_bf16(const bf16_t* A, const bf16_t* Wp, void* out, int out_is_f32, int 
         default: return fail(SD3_ERR_INVALID_ARG, "gemm_bf16: unknown epilogue %d", epi);
     }
 #undef SD3_GEMM_BF16_LAUNCH
+}
+
+int gemm_bf16(const bf16_t* A, const bf16_t* Wp, void* out, int out_is_f32, int ldc, int M, int N, int K, int epi, const GemmEpilogueArgs& ea,
+              hipStream_t st) {
+    GemmBf16Problem q{A, Wp, out, ldc, M, N, K, ea};
+    return gemm_bf16_grouped(&q, 1, out_is_f32, epi, st);
 }
 
 }  // namespace sd3
