@@ -14,6 +14,9 @@ LIB = os.path.join(HERE, "libsd3_hip.so")
 SOURCES = ["pointwise.hip", "small_linear.hip", "gemm_f32.hip", "gemm_bf16.hip", "attention_f32.hip", "attention_bf16.hip", "engine.hip"]
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-sanitize", "-Wall", "-Wno-unused-function",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+# the attention kernel's running-maximum chains carry no NaNs by construction; without this flag every fmaxf is preceded
+# by a canonicalising v_max of each operand
+EXTRA_FLAGS = {"attention_bf16.hip": ["-fno-honor-nans"]}
 DEPS = [os.path.join(CSRC, "common.hpp"), os.path.join(os.path.dirname(HERE), "include", "sd3_hip.h")]
 
 
@@ -28,7 +31,7 @@ def _compile(src, force):
     obj = os.path.join(OBJ, src.replace(".hip", ".o"))
     path = os.path.join(CSRC, src)
     if force or _stale(obj, [path] + DEPS):
-        r = subprocess.run(["hipcc"] + FLAGS + ["-c", path, "-o", obj], capture_output=True, text=True)
+        r = subprocess.run(["hipcc"] + FLAGS + EXTRA_FLAGS.get(src, []) + ["-c", path, "-o", obj], capture_output=True, text=True)
         # the host pass does not know the packed-fp32 feature flag and says so once per pass; that line is noise
         err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l)
         if r.returncode != 0:

@@ -1,26 +1,37 @@
 // Joint text+image flash attention for head_dim 64 on the gfx950 bf16 matrix cores (v_mfma_f32_32x32x16_bf16).
 //
 // One launch does what the reference does in eight calls (modules.cpp:1396-1399, 1420-1432): per-head RMSNorm of q
-// and k (applied while the operands are loaded), concatenation of context and latent tokens (never materialised:
-// rows of the joint sequence are fetched from the context buffer below T[0] and from the latent buffer above),
-// softmax(q k^T / sqrt(64)) v with an online softmax (no T x T matrix), and the split of the result.
+// and k (optional: applied while the operands are loaded), concatenation of context and latent tokens (never
+// materialised: rows of the joint sequence are fetched from the context buffer below T[0] and from the latent buffer
+// above), softmax(q k^T / sqrt(64)) v with an online softmax (no T x T matrix), and the split of the result.
 // q, k, v are the column thirds of the packed (tokens, 3C) bf16 buffers that the QKV GEMM writes; head h is columns
 // [h*64, h*64+64) inside a third, exactly the reference's layout.
 //
 // Everything is kept transposed so that probabilities stay in registers between the two matrix products:
-//   S^T (keys x queries) = K . Q^T     : a lane owns one query column and 16 of every 32 keys
+//   S^T (keys x queries) = K . Q^T     : a lane owns one query column per 32-query block and 16 of every 32 keys
 //   O^T (d x queries)   += V^T . P^T   : the lane's S^T registers 8j..8j+7 are, unchanged, the P^T operand of step j
 // which needs V^T (d-major) in LDS; V rows are transposed while being staged (two keys packed per 32-bit store).
+// A wavefront owns 64 queries (two 32-query blocks), so every K / V^T fragment read from LDS feeds two matrix
+// instructions; a workgroup of 4 wavefronts shares each 64-key tile. K tiles go global -> LDS directly
+// (global_load_lds_dwordx4) into 128-byte rows with XOR-swizzled 16-byte chunks; tiles are double-buffered with one
+// barrier per tile.
 #include "common.hpp"
 
 namespace sd3 {
 namespace {
 
 constexpr int HS = 64;
-constexpr int BQ = 128;       // queries per workgroup: 4 wavefronts x 32
-constexpr int BKV = 64;       // keys per tile
-constexpr int K_PITCH = 72;   // bf16 per K row in LDS (144 B: conflict-free 16-byte reads across 16 rows)
-constexpr int V_PITCH = 66;   // bf16 per V^T row (33 words: conflict-free transposing stores and 8-byte reads)
+constexpr int NW = 4;            // wavefronts per workgroup
+constexpr int QW = 64;           // queries per wavefront
+constexpr int BQ = NW * QW;      // queries per workgroup
+constexpr int BKV = 64;          // keys per tile
+constexpr int V_PITCH = 66;      // bf16 per V^T row (33 words: conflict-free transposing stores and 8-byte reads)
+constexpr int K_BYTES = BKV * 128, V_BYTES = HS * V_PITCH * 2, STAGE_BYTES = K_BYTES + V_BYTES;
+constexpr int O_PITCH = 72;      // bf16 per staged output row
+constexpr int SMEM_BYTES = (2 * STAGE_BYTES > NW * QW * O_PITCH * 2) ? 2 * STAGE_BYTES : NW * QW * O_PITCH * 2;
+
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+typedef const __attribute__((address_space(1))) void* glb_ptr_t;
 
 struct SegDev {
     const bf16_t* q[2];
@@ -33,7 +44,10 @@ struct SegDev {
     int ld_out[2];
     int T[2];
     int Tq[2];
+    int NH, nqb;  // heads, query blocks per (batch, head)
 };
+
+__device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 1); }
 
 __device__ __forceinline__ void unpack8(const uint4& u, float (&f)[8]) {
     f[0] = __uint_as_float(u.x << 16); f[1] = __uint_as_float(u.x & 0xffff0000u);
@@ -49,22 +63,35 @@ union Frag {
     bf16x8_t v;
 };
 
-__global__ void __launch_bounds__(256) flash_attn_bf16_kernel(SegDev s, float q_scale /* log2(e)/sqrt(64) */, float eps) {
-    // K tile (64 x 72) and V^T tile (64 x 66); the same memory later holds the output tile (128 x 72)
-    __shared__ __attribute__((aligned(16))) bf16_t smem[BQ * K_PITCH];
-    static_assert(BKV * K_PITCH + HS * V_PITCH <= BQ * K_PITCH, "tiles must fit the shared buffer");
-    bf16_t* const Ks = smem;
-    bf16_t* const Vt = smem + BKV * K_PITCH;
+// NORM: apply the per-head RMSNorm to q and k while loading them (K then goes through registers instead of the
+// direct global->LDS path). Without it q and k are taken as they are (already normalised by the QKV GEMM epilogue).
+template <bool NORM>
+__global__ void __launch_bounds__(NW * 64, 2) flash_attn_bf16_kernel(SegDev s, float q_scale /* log2(e)/sqrt(64) */, float eps) {
+    __shared__ __attribute__((aligned(1024))) char smem[SMEM_BYTES];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int l32 = lane & 31, lk = lane >> 5;
-    const int h = blockIdx.y, b = blockIdx.z;
     const int T0 = s.T[0], T = s.T[0] + s.T[1];
     const int Tq0 = s.Tq[0], TQ = s.Tq[0] + s.Tq[1];
 
-    // ---- Q^T operand: lane = query l32 of this wavefront; k-step ks covers d = 16*ks + 8*lk + (0..7) ----
-    const int qt = blockIdx.x * BQ + wave * 32 + l32;
-    Frag qf[4];
+    // ---- workgroup -> (batch, head, query block): consecutive workgroup ids go to different XCDs (each with its own L2),
+    //      so the workgroups of one XCD get a contiguous run of work items; all query blocks of a head then share K/V in one L2
+    int b, h, qblk;
     {
+        const int total = gridDim.x, wg = blockIdx.x, xcd = wg % 8, local = wg / 8;
+        const int per = (total + 7) / 8, tall = (total % 8) ? (total % 8) : 8;
+        const int t = (xcd < tall) ? xcd * per + local : tall * per + (xcd - tall) * (per - 1) + local;
+        const int bh = t / s.nqb;
+        qblk = t % s.nqb;
+        b = bh / s.NH;
+        h = bh % s.NH;
+    }
+
+    // ---- Q^T operands: for block qb the lane is query (q0 + 32 qb + l32); k-step ks covers d = 16 ks + 8 lk + (0..7) ----
+    const int q0 = qblk * BQ + wave * QW;
+    Frag qf[2][4];
+#pragma unroll
+    for (int qb = 0; qb < 2; qb++) {
+        const int qt = q0 + qb * 32 + l32;
         const int seg = (qt < Tq0) ? 0 : 1;
         float f[4][8];
         float ss = 0.f;
@@ -74,8 +101,9 @@ __global__ void __launch_bounds__(256) flash_attn_bf16_kernel(SegDev s, float q_
             for (int ks = 0; ks < 4; ks++) {
                 const uint4 u = *reinterpret_cast<const uint4*>(qp + ks * 16 + lk * 8);
                 unpack8(u, f[ks]);
+                if (NORM)
 #pragma unroll
-                for (int e = 0; e < 8; e++) ss += f[ks][e] * f[ks][e];
+                    for (int e = 0; e < 8; e++) ss += f[ks][e] * f[ks][e];
             }
         } else {
 #pragma unroll
@@ -83,176 +111,226 @@ __global__ void __launch_bounds__(256) flash_attn_bf16_kernel(SegDev s, float q_
 #pragma unroll
                 for (int e = 0; e < 8; e++) f[ks][e] = 0.f;
         }
-        ss += __shfl_xor(ss, 32, 64);  // the other half of the row lives in lane ^ 32
-        const float* w = s.rms_q[seg];
-        const float mul = w ? q_scale / sqrtf(eps + ss * (1.0f / HS)) : q_scale;
+        const float* w = NORM ? s.rms_q[seg] : nullptr;
+        float mul = q_scale;
+        if (NORM) {
+            ss += __shfl_xor(ss, 32, 64);  // the other half of the row lives in lane ^ 32
+            if (w) mul = q_scale / sqrtf(eps + ss * (1.0f / HS));
+        }
 #pragma unroll
         for (int ks = 0; ks < 4; ks++) {
 #pragma unroll
-            for (int e = 0; e < 8; e++) f[ks][e] *= w ? mul * w[ks * 16 + lk * 8 + e] : mul;
-            qf[ks].u = pack8(f[ks]);
+            for (int e = 0; e < 8; e++) f[ks][e] *= (NORM && w) ? mul * w[ks * 16 + lk * 8 + e] : mul;
+            qf[qb][ks].u = pack8(f[ks]);
         }
     }
 
-    f32x16_t oacc[2];
+    f32x16_t oacc[2][2];  // [d block][query block]
 #pragma unroll
     for (int i = 0; i < 2; i++)
 #pragma unroll
-        for (int r = 0; r < 16; r++) oacc[i][r] = 0.f;
-    float m_run = -1e30f, l_run = 0.f;
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) oacc[i][j][r] = 0.f;
+    float m_run[2] = {-1e30f, -1e30f}, l_run[2] = {0.f, 0.f};
+    constexpr float TAU = 8.0f;
+    const bf16x2_t ONES = {(__bf16)1.0f, (__bf16)1.0f};
 
     // ---- staging roles ----
-    // K: 64 rows x 8 chunks of 16 B = 512 chunks, 2 per thread (rows r and r+32); 8 consecutive lanes share a row
-    const int k_row = tid >> 3, k_ch = tid & 7;
-    // V: thread = (key pair, d-chunk): rows 2*vp and 2*vp+1, d = 8*v_ch..+7; stored transposed, two keys per 32-bit word
-    const int v_pair = tid >> 3, v_ch = tid & 7;
-    uint4 rk[2], rv[2];
     auto kv_row_ptr = [&](const bf16_t* const* base, int t) -> const bf16_t* {
+        t = min(t, T - 1);  // rows beyond the sequence re-read the last row: finite values, masked out of the softmax below
         const int seg = (t < T0) ? 0 : 1;
         return base[seg] + ((long long)b * s.T[seg] + (seg ? t - T0 : t)) * s.ld_qkv[seg] + h * HS;
     };
-    auto load_kv = [&](int t0) {
+    // K: chunk q = i*256 + tid of the tile lands at LDS byte q*16 (row q/8, physical chunk q%8, logical chunk XOR-swizzled)
+    // V: thread = (key pair, d-chunk): rows 2*vp and 2*vp+1, d = 8*v_ch..+7; stored transposed, two keys per 32-bit word
+    const int v_pair = tid >> 3, v_ch = tid & 7;
+    uint4 rk[2], rv[2];
+    // Row pointers of this thread's two K chunks and two V rows. Inside a segment they advance by a constant per tile;
+    // they are recomputed from scratch only for the first tile, the tiles around the segment boundary and the last tile.
+    const bf16_t* kp[2];
+    const bf16_t* vp[2];
+    auto issue_tile = [&](int t0, int stage) {
+        char* ks_ = smem + stage * STAGE_BYTES;
+        const bool in0 = (t0 >= BKV) && (t0 + BKV <= T0), in1 = (t0 - BKV >= T0) && (t0 + BKV <= T);
+        if (in0 || in1) {
+            const long long step = (long long)BKV * s.ld_qkv[in1 ? 1 : 0];
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+                kp[i] += step;
+                vp[i] += step;
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+                const int q = i * 256 + tid, row = q >> 3, lc = (q & 7) ^ swz(row);
+                kp[i] = kv_row_ptr(s.k, t0 + row) + lc * 8;
+                vp[i] = kv_row_ptr(s.v, t0 + 2 * v_pair + i) + v_ch * 8;
+            }
+        }
 #pragma unroll
         for (int i = 0; i < 2; i++) {
-            const int tk = t0 + k_row + i * 32;
-            rk[i] = (tk < T) ? *reinterpret_cast<const uint4*>(kv_row_ptr(s.k, tk) + k_ch * 8) : make_uint4(0, 0, 0, 0);
-            const int tv = t0 + 2 * v_pair + i;
-            rv[i] = (tv < T) ? *reinterpret_cast<const uint4*>(kv_row_ptr(s.v, tv) + v_ch * 8) : make_uint4(0, 0, 0, 0);
+            if (NORM) rk[i] = *reinterpret_cast<const uint4*>(kp[i]);
+            else __builtin_amdgcn_global_load_lds((glb_ptr_t)kp[i], (lds_ptr_t)(ks_ + (i * 256 + wave * 64) * 16), 16, 0, 0);
+            rv[i] = *reinterpret_cast<const uint4*>(vp[i]);
         }
     };
-    auto store_kv = [&](int t0) {
+    auto store_tile = [&](int t0, int stage) {
+        char* ks_ = smem + stage * STAGE_BYTES;
+        if (NORM) {
 #pragma unroll
-        for (int i = 0; i < 2; i++) {
-            const int tk = t0 + k_row + i * 32;
-            const float* w = s.rms_k[(tk < T0) ? 0 : 1];
-            uint4 u = rk[i];
-            if (w) {
-                float f[8];
-                unpack8(u, f);
-                float ss = 0.f;
+            for (int i = 0; i < 2; i++) {
+                const int q = i * 256 + tid, row = q >> 3, lc = (q & 7) ^ swz(row);
+                const float* w = s.rms_k[(min(t0 + row, T - 1) < T0) ? 0 : 1];
+                uint4 u = rk[i];
+                if (w) {
+                    float f[8];
+                    unpack8(u, f);
+                    float ss = 0.f;
 #pragma unroll
-                for (int e = 0; e < 8; e++) ss += f[e] * f[e];
-                ss += __shfl_xor(ss, 1, 64);
-                ss += __shfl_xor(ss, 2, 64);
-                ss += __shfl_xor(ss, 4, 64);
-                const float inv = 1.0f / sqrtf(eps + ss * (1.0f / HS));
+                    for (int e = 0; e < 8; e++) ss += f[e] * f[e];
+                    ss += __shfl_xor(ss, 1, 64);  // the 8 chunks of a row sit in 8 consecutive lanes
+                    ss += __shfl_xor(ss, 2, 64);
+                    ss += __shfl_xor(ss, 4, 64);
+                    const float inv = 1.0f / sqrtf(eps + ss * (1.0f / HS));
 #pragma unroll
-                for (int e = 0; e < 8; e++) f[e] *= inv * w[k_ch * 8 + e];
-                u = pack8(f);
+                    for (int e = 0; e < 8; e++) f[e] *= inv * w[lc * 8 + e];
+                    u = pack8(f);
+                }
+                *reinterpret_cast<uint4*>(ks_ + q * 16) = u;
             }
-            *reinterpret_cast<uint4*>(&Ks[(k_row + i * 32) * K_PITCH + k_ch * 8]) = u;
         }
         // V^T[d][2*vp .. 2*vp+1] = (V[2vp][d], V[2vp+1][d])
         const uint32_t a[4] = {rv[0].x, rv[0].y, rv[0].z, rv[0].w};
         const uint32_t c[4] = {rv[1].x, rv[1].y, rv[1].z, rv[1].w};
-        uint32_t* vt32 = reinterpret_cast<uint32_t*>(Vt);
+        uint32_t* vt32 = reinterpret_cast<uint32_t*>(ks_ + K_BYTES);
 #pragma unroll
         for (int e = 0; e < 4; e++) {
-            const uint32_t lo = (a[e] & 0xffffu) | (c[e] << 16);          // d = 8*v_ch + 2e
-            const uint32_t hi = (a[e] >> 16) | (c[e] & 0xffff0000u);      // d = 8*v_ch + 2e + 1
-            vt32[((v_ch * 8 + 2 * e) * V_PITCH) / 2 + v_pair] = lo;
-            vt32[((v_ch * 8 + 2 * e + 1) * V_PITCH) / 2 + v_pair] = hi;
+            vt32[((v_ch * 8 + 2 * e) * V_PITCH) / 2 + v_pair] = (a[e] & 0xffffu) | (c[e] << 16);            // d = 8*v_ch + 2e
+            vt32[((v_ch * 8 + 2 * e + 1) * V_PITCH) / 2 + v_pair] = (a[e] >> 16) | (c[e] & 0xffff0000u);    // d = 8*v_ch + 2e + 1
         }
     };
 
-    load_kv(0);
-    for (int t0 = 0; t0 < T; t0 += BKV) {
-        __syncthreads();  // the previous tile has been consumed by every wavefront
-        store_kv(t0);
-        __syncthreads();
-        if (t0 + BKV < T) load_kv(t0 + BKV);  // in flight during the matrix work below
+    const int nt = (T + BKV - 1) / BKV;
+    issue_tile(0, 0);
+    store_tile(0, 0);
+    const int ksw = swz(l32);
 
-        // ---- S^T = K . Q^T for the two 32-key blocks ----
-        f32x16_t sacc[2];
+    for (int t = 0; t < nt; t++) {
+        __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8));  // vmcnt(0): this thread's direct K loads of tile t have landed
+        __syncthreads();  // tile t is complete in LDS, and every wavefront is done reading the other stage
+        const bool more = t + 1 < nt;
+        if (more) issue_tile((t + 1) * BKV, (t + 1) & 1);
+        const char* ks_ = smem + (t & 1) * STAGE_BYTES;
+        const bf16_t* vt = reinterpret_cast<const bf16_t*>(ks_ + K_BYTES);
+
 #pragma unroll
-        for (int kb = 0; kb < 2; kb++) {
-#pragma unroll
-            for (int r = 0; r < 16; r++) sacc[kb][r] = 0.f;
+        for (int kb = 0; kb < 2; kb++) {  // two 32-key halves of the tile
+            // ---- S^T = K . Q^T : one K fragment feeds both query blocks ----
+            f32x16_t sacc[2];
+            const f32x16_t zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int ks = 0; ks < 4; ks++) {
-                const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(&Ks[(kb * 32 + l32) * K_PITCH + ks * 16 + lk * 8]);
-                sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[ks].v, sacc[kb], 0, 0, 0);
-            }
-        }
-        // ---- online softmax (base 2: log2(e)/8 is folded into q). Register r of block kb is key t0+32kb+8(r/4)+4lk+r%4 ----
-        if (t0 + BKV > T) {
+                const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(ks_ + (kb * 32 + l32) * 128 + (((2 * ks + lk) ^ ksw) * 16));
 #pragma unroll
-            for (int kb = 0; kb < 2; kb++)
+                for (int qb = 0; qb < 2; qb++) sacc[qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[qb][ks].v, ks == 0 ? zero : sacc[qb], 0, 0, 0);
+            }
+            // register r is key  t*64 + 32 kb + 8 (r/4) + 4 lk + r%4
+            if (t == nt - 1) {
+                const int kbase = t * BKV + kb * 32 + 4 * lk;
 #pragma unroll
                 for (int r = 0; r < 16; r++)
-                    if (t0 + kb * 32 + 8 * (r >> 2) + 4 * lk + (r & 3) >= T) sacc[kb][r] = -1e30f;
-        }
-        float tmax = sacc[0][0];
-#pragma unroll
-        for (int kb = 0; kb < 2; kb++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) tmax = fmaxf(tmax, sacc[kb][r]);
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-        const float m_new = fmaxf(m_run, tmax);
-        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-        m_run = m_new;
-        float psum = 0.f;
-#pragma unroll
-        for (int kb = 0; kb < 2; kb++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const float p = __builtin_amdgcn_exp2f(sacc[kb][r] - m_new);
-                sacc[kb][r] = p;
-                psum += p;
+                    if (kbase + 8 * (r >> 2) + (r & 3) >= T) {
+                        sacc[0][r] = -1e30f;
+                        sacc[1][r] = -1e30f;
+                    }
             }
-        l_run = l_run * alpha + psum;
-        if (__any(alpha != 1.0f)) {  // once the running maxima have settled no lane needs the rescale
+            // ---- online softmax per query block (base 2: log2(e)/8 is folded into q). The reference maximum m_run is only
+            //      raised when some score exceeds it by more than 2^TAU (probabilities then stay below 2^TAU, harmless in
+            //      fp32 / bf16), so the accumulator rescale runs on the first tile and hardly ever after that. ----
+            Frag pf[2][2];
 #pragma unroll
-            for (int i = 0; i < 2; i++)
+            for (int qb = 0; qb < 2; qb++) {
+                float tmax = fmaxf(sacc[qb][0], sacc[qb][1]);
 #pragma unroll
-                for (int r = 0; r < 16; r++) oacc[i][r] *= alpha;
-        }
-
-        // ---- O^T += V^T . P^T ; step j of block kb contracts keys 32kb + 16j + {4lk..4lk+3, 8+4lk..8+4lk+3} ----
+                for (int r = 2; r < 16; r += 2) tmax = fmaxf(tmax, fmaxf(sacc[qb][r], sacc[qb][r + 1]));
+                if (__any(tmax > m_run[qb] + TAU)) {
+                    // lanes l and l^32 hold the two key halves of the same query and feed the same accumulators: same reference
+                    const float m_new = fmaxf(m_run[qb], fmaxf(tmax, __shfl_xor(tmax, 32, 64)));
+                    const float alpha = __builtin_amdgcn_exp2f(m_run[qb] - m_new);
+                    m_run[qb] = m_new;
+                    l_run[qb] *= alpha;
 #pragma unroll
-        for (int kb = 0; kb < 2; kb++)
+                    for (int db = 0; db < 2; db++)
+#pragma unroll
+                        for (int r = 0; r < 16; r++) oacc[db][qb][r] *= alpha;
+                }
+                const float mref = m_run[qb];
+#pragma unroll
+                for (int r = 0; r < 16; r++) sacc[qb][r] = __builtin_amdgcn_exp2f(sacc[qb][r] - mref);
+                float ls0 = l_run[qb], ls1 = 0.f;
+#pragma unroll
+                for (int j = 0; j < 2; j++) {
+                    uint32_t w[4];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        w[e] = pack_bf16x2(sacc[qb][8 * j + 2 * e], sacc[qb][8 * j + 2 * e + 1]);
+                        // row sum of the rounded probabilities, two per instruction
+                        if (e & 1) ls1 = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, w[e]), ONES, ls1, false);
+                        else ls0 = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, w[e]), ONES, ls0, false);
+                    }
+                    pf[qb][j].u = make_uint4(w[0], w[1], w[2], w[3]);
+                }
+                l_run[qb] = ls0 + ls1;
+            }
+            // ---- O^T += V^T . P^T ; step j contracts keys 32kb + 16j + {4lk..4lk+3, 8+4lk..8+4lk+3}; one V^T fragment feeds both query blocks ----
 #pragma unroll
             for (int j = 0; j < 2; j++) {
-                Frag pf;
-                pf.u = make_uint4(pack_bf16x2(sacc[kb][8 * j + 0], sacc[kb][8 * j + 1]), pack_bf16x2(sacc[kb][8 * j + 2], sacc[kb][8 * j + 3]),
-                                  pack_bf16x2(sacc[kb][8 * j + 4], sacc[kb][8 * j + 5]), pack_bf16x2(sacc[kb][8 * j + 6], sacc[kb][8 * j + 7]));
                 const int key0 = kb * 32 + 16 * j + 4 * lk;
 #pragma unroll
                 for (int db = 0; db < 2; db++) {
-                    const uint32_t* row = reinterpret_cast<const uint32_t*>(&Vt[(db * 32 + l32) * V_PITCH + key0]);
+                    const uint32_t* row = reinterpret_cast<const uint32_t*>(&vt[(db * 32 + l32) * V_PITCH + key0]);
                     Frag vf;
                     vf.u = make_uint4(row[0], row[1], row[4], row[5]);
-                    oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf.v, pf.v, oacc[db], 0, 0, 0);
+#pragma unroll
+                    for (int qb = 0; qb < 2; qb++) oacc[db][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf.v, pf[qb][j].v, oacc[db][qb], 0, 0, 0);
                 }
             }
+        }
+        if (more) store_tile((t + 1) * BKV, (t + 1) & 1);
     }
 
-    // ---- normalise; transpose through LDS (reusing the K tile) so that rows leave as 16-byte stores ----
-    const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
-    const float inv = 1.0f / l_tot;
+    // ---- normalise; transpose through LDS (each wavefront its own 64-row region) so that rows leave as 16-byte stores ----
     __syncthreads();
-    bf16_t* Ow = smem + wave * 32 * K_PITCH;  // this wavefront's 32 output rows
+    bf16_t* Ow = reinterpret_cast<bf16_t*>(smem) + wave * QW * O_PITCH;
 #pragma unroll
-    for (int db = 0; db < 2; db++)
+    for (int qb = 0; qb < 2; qb++) {
+        const float l_tot = l_run[qb] + __shfl_xor(l_run[qb], 32, 64);
+        const float inv = 1.0f / l_tot;
 #pragma unroll
-        for (int g = 0; g < 4; g++) {
-            const int d0 = db * 32 + 8 * g + 4 * lk;
-            const uint2 v = make_uint2(pack_bf16x2(oacc[db][4 * g + 0] * inv, oacc[db][4 * g + 1] * inv),
-                                       pack_bf16x2(oacc[db][4 * g + 2] * inv, oacc[db][4 * g + 3] * inv));
-            *reinterpret_cast<uint2*>(&Ow[l32 * K_PITCH + d0]) = v;
-        }
-    __syncthreads();
-    // 32 rows x 8 chunks per wavefront = 256 chunks, 4 per lane
+        for (int db = 0; db < 2; db++)
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
+            for (int g = 0; g < 4; g++) {
+                const int d0 = db * 32 + 8 * g + 4 * lk;
+                const uint2 v = make_uint2(pack_bf16x2(oacc[db][qb][4 * g + 0] * inv, oacc[db][qb][4 * g + 1] * inv),
+                                           pack_bf16x2(oacc[db][qb][4 * g + 2] * inv, oacc[db][qb][4 * g + 3] * inv));
+                *reinterpret_cast<uint2*>(&Ow[(qb * 32 + l32) * O_PITCH + d0]) = v;
+            }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    // 64 rows x 8 chunks per wavefront = 512 chunks, 8 per lane
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
         const int c = lane + i * 64;
         const int row = c >> 3, ch = c & 7;
-        const int t = blockIdx.x * BQ + wave * 32 + row;
+        const int t = q0 + row;
         if (t < TQ) {
             const int seg = (t < Tq0) ? 0 : 1;
             if (s.out[seg]) {
                 bf16_t* op = s.out[seg] + ((long long)b * s.Tq[seg] + (seg ? t - Tq0 : t)) * s.ld_out[seg] + h * HS + ch * 8;
-                *reinterpret_cast<uint4*>(op) = *reinterpret_cast<const uint4*>(&Ow[row * K_PITCH + ch * 8]);
+                *reinterpret_cast<uint4*>(op) = *reinterpret_cast<const uint4*>(&Ow[row * O_PITCH + ch * 8]);
             }
         }
     }
@@ -266,6 +344,7 @@ int attention_bf16(const AttnSegments& a, int B, int NH, int hs, hipStream_t st)
     if (hs != HS) return fail(SD3_ERR_UNSUPPORTED, "attention (bf16): head_dim must be 64 (got %d)", hs);
     if (T <= 0) return fail(SD3_ERR_INVALID_ARG, "attention: no keys");
     SegDev s;
+    bool norm = false;
     for (int i = 0; i < 2; i++) {
         s.q[i] = (const bf16_t*)a.q[i]; s.k[i] = (const bf16_t*)a.k[i]; s.v[i] = (const bf16_t*)a.v[i]; s.out[i] = (bf16_t*)a.out[i];
         s.rms_q[i] = a.rms_q[i]; s.rms_k[i] = a.rms_k[i];
@@ -276,11 +355,15 @@ int attention_bf16(const AttnSegments& a, int B, int NH, int hs, hipStream_t st)
             if ((a.ld_qkv[i] % 8) || (a.ld_out[i] % 8) || (reinterpret_cast<uintptr_t>(a.q[i]) & 15) || (reinterpret_cast<uintptr_t>(a.k[i]) & 15) ||
                 (reinterpret_cast<uintptr_t>(a.v[i]) & 15) || (reinterpret_cast<uintptr_t>(a.out[i]) & 15))
                 return fail(SD3_ERR_INVALID_ARG, "attention (bf16): rows must be 16-byte aligned (segment %d)", i);
+            if (a.rms_q[i] || a.rms_k[i]) norm = true;
         }
     }
+    s.NH = NH;
+    s.nqb = (TQ + BQ - 1) / BQ;
     const float q_scale = 1.4426950408889634f / sqrtf((float)HS);
-    dim3 grid((TQ + BQ - 1) / BQ, NH, B), block(256);
-    hipLaunchKernelGGL(flash_attn_bf16_kernel, grid, block, 0, st, s, q_scale, 1e-6f);
+    dim3 grid((unsigned)(s.nqb * NH * B)), block(NW * 64);
+    if (norm) hipLaunchKernelGGL(flash_attn_bf16_kernel<true>, grid, block, 0, st, s, q_scale, 1e-6f);
+    else hipLaunchKernelGGL(flash_attn_bf16_kernel<false>, grid, block, 0, st, s, q_scale, 1e-6f);
     return launch_status("flash_attention_bf16");
 }
 

@@ -87,6 +87,8 @@ enum Epilogue : int {
     EPI_BIAS_SILU = 2,    // out = silu(acc + bias)
     EPI_GATE_RESID = 3,   // out = resid + gate[m / rows_per_batch][n] * (acc + bias)   (out may alias resid)
     EPI_BIAS_ROWADD = 4,  // out = acc + bias + table[m % rows_per_batch][n]
+    EPI_QKV_NORM = 5,     // packed q|k|v projection (N = 3C): acc + bias, then per-head RMSNorm (64 columns, eps 1e-6) of the q and k thirds
+                          // with weights `gate` (q) and `resid` (k), each 64 floats; C is given in gate_ld
 };
 
 struct GemmEpilogueArgs {

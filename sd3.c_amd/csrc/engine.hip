@@ -308,11 +308,18 @@ int run_block(sd3_ctx* ctx, int prec, const float* y, float* c, float* x, const 
     SD3_TRY(ln_mod(ctx, x, x_hid, d.dual ? x_hid2 : nullptr, xchunk(0), xchunk(1), d.dual ? xchunk(6) : nullptr, d.dual ? xchunk(7) : nullptr, ldx_ada,
                    1e-6f, B, Tx, C, bf));
     {
-        LayerCall qkv[2] = {{x_hid, w.x_qkv_w, w.x_qkv_b, x_qkv, 3 * C, mx, 3 * C, C, none}, {c_hid, w.c_qkv_w, w.c_qkv_b, c_qkv, 3 * C, mc, 3 * C, C, none}};
-        SD3_TRY(linear_pair(ctx, prec, qkv, 2, !bf, EPI_BIAS));
+        // bf16 path: the per-head RMSNorm of q and k (modules.cpp:1396-1399, 1420-1423) runs in the projection's epilogue, on the
+        // fp32 accumulators, so the attention kernel streams K tiles straight into LDS
+        GemmEpilogueArgs nx, nc;
+        nx.gate = w.x_rms_q; nx.resid = w.x_rms_k;
+        nc.gate = w.c_rms_q; nc.resid = w.c_rms_k;
+        const bool fused_norm = bf && d.qk;
+        LayerCall qkv[2] = {{x_hid, w.x_qkv_w, w.x_qkv_b, x_qkv, 3 * C, mx, 3 * C, C, fused_norm ? nx : none},
+                            {c_hid, w.c_qkv_w, w.c_qkv_b, c_qkv, 3 * C, mc, 3 * C, C, fused_norm ? nc : none}};
+        SD3_TRY(linear_pair(ctx, prec, qkv, 2, !bf, fused_norm ? EPI_QKV_NORM : EPI_BIAS));
     }
 
-    // ---- joint attention over [context ; latent] (modules.cpp:1427-1432), qk-norm fused (bf16) or done in place first (fp32)
+    // ---- joint attention over [context ; latent] (modules.cpp:1427-1432); fp32 path: qk-norm in place first
     auto seg_ptr = [&](void* base, int third) -> void* { return (char*)base + (size_t)third * C * es; };
     if (!bf && d.qk) {
         SD3_TRY(rmsnorm_rows((float*)c_qkv, (float*)c_qkv, w.c_rms_q, nullptr, 1e-6f, mc, d.NH, d.HS, 3 * C, 3 * C, st));
@@ -326,8 +333,7 @@ int run_block(sd3_ctx* ctx, int prec, const float* y, float* c, float* x, const 
         a.q[1] = x_qkv; a.k[1] = seg_ptr(x_qkv, 1); a.v[1] = seg_ptr(x_qkv, 2); a.out[1] = x_att;
         a.ld_qkv[0] = a.ld_qkv[1] = 3 * C; a.ld_out[0] = a.ld_out[1] = C;
         a.T[0] = a.Tq[0] = Tc; a.T[1] = a.Tq[1] = Tx;
-        if (d.qk) { a.rms_q[0] = w.c_rms_q; a.rms_k[0] = w.c_rms_k; a.rms_q[1] = w.x_rms_q; a.rms_k[1] = w.x_rms_k; }
-        SD3_TRY(attention(ctx, a, B, d.NH, d.HS, bf));
+        SD3_TRY(attention(ctx, a, B, d.NH, d.HS, bf));  // q and k arrive normalised on both paths
     }
     // ---- out-projections with the gate and the residual add in the epilogue (modules.cpp:1435-1436, 1459-1462, 1481-1485)
     GemmEpilogueArgs gx, gc;
@@ -340,7 +346,10 @@ int run_block(sd3_ctx* ctx, int prec, const float* y, float* c, float* x, const 
 
     // ---- extra self-attention over the latent tokens (modules.cpp:1440-1453, 1486)
     if (d.dual) {
-        SD3_TRY(linear_layer(ctx, prec, x_hid2, w.x2_qkv_w, w.x2_qkv_b, x_qkv, !bf, 3 * C, mx, 3 * C, C, EPI_BIAS, none));
+        GemmEpilogueArgs n2;
+        n2.gate = w.x2_rms_q; n2.resid = w.x2_rms_k;
+        SD3_TRY(linear_layer(ctx, prec, x_hid2, w.x2_qkv_w, w.x2_qkv_b, x_qkv, !bf, 3 * C, mx, 3 * C, C, (bf && d.qk) ? EPI_QKV_NORM : EPI_BIAS,
+                             (bf && d.qk) ? n2 : none));
         if (!bf && d.qk) {
             SD3_TRY(rmsnorm_rows((float*)x_qkv, (float*)x_qkv, w.x2_rms_q, nullptr, 1e-6f, mx, d.NH, d.HS, 3 * C, 3 * C, st));
             SD3_TRY(rmsnorm_rows((float*)seg_ptr(x_qkv, 1), (float*)seg_ptr(x_qkv, 1), w.x2_rms_k, nullptr, 1e-6f, mx, d.NH, d.HS, 3 * C, 3 * C, st));
@@ -349,7 +358,6 @@ int run_block(sd3_ctx* ctx, int prec, const float* y, float* c, float* x, const 
         a.q[0] = x_qkv; a.k[0] = seg_ptr(x_qkv, 1); a.v[0] = seg_ptr(x_qkv, 2); a.out[0] = x_att;
         a.ld_qkv[0] = a.ld_qkv[1] = 3 * C; a.ld_out[0] = a.ld_out[1] = C;
         a.T[0] = a.Tq[0] = Tx;
-        if (d.qk) { a.rms_q[0] = w.x2_rms_q; a.rms_k[0] = w.x2_rms_k; }
         SD3_TRY(attention(ctx, a, B, d.NH, d.HS, bf));
         GemmEpilogueArgs g2;
         g2.rows_per_batch = Tx; g2.gate = xchunk(8); g2.gate_ld = ldx_ada; g2.resid = x;

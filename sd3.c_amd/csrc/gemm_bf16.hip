@@ -245,6 +245,21 @@ __global__ void __launch_bounds__(WM* WN * 64) gemm_bf16_kernel(const ProbPair a
                     for (int c = 0; c < 4; c++)
                         if (c < nvalid) v[c] += t[c];
                 }
+                if (EPI == EPI_QKV_NORM) {
+                    // the 16 lanes that hold this row's 64 columns are one head of one token (modules.cpp:192-198, fused)
+                    static_assert(EPI != EPI_QKV_NORM || WNC == 64, "the fused qk-norm needs one head per wavefront slab");
+                    const int third = (n_blk + wn * WNC) / epi.gate_ld;  // 0 = q, 1 = k, 2 = v (wavefront-uniform)
+                    if (third < 2) {
+                        float ss = (v[0] * v[0] + v[1] * v[1]) + (v[2] * v[2] + v[3] * v[3]);
+                        ss += __shfl_xor(ss, 1, 64);
+                        ss += __shfl_xor(ss, 2, 64);
+                        ss += __shfl_xor(ss, 4, 64);
+                        ss += __shfl_xor(ss, 8, 64);
+                        const float inv = 1.0f / sqrtf(1e-6f + ss * (1.0f / 64.0f));
+                        const float4 w4 = *reinterpret_cast<const float4*>((third == 0 ? epi.gate : epi.resid) + e_col);
+                        v[0] *= inv * w4.x; v[1] *= inv * w4.y; v[2] *= inv * w4.z; v[3] *= inv * w4.w;
+                    }
+                }
                 if (vec_ok) {
                     if (OUT_F32) *reinterpret_cast<float4*>(outf + idx) = make_float4(v[0], v[1], v[2], v[3]);
                     else *reinterpret_cast<uint2*>(outh + idx) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
@@ -282,8 +297,6 @@ int launch_cfg(ProbPair& args, int n, hipStream_t st) {
 template <int EPI, bool OUT_F32>
 int launch_epi(int variant, ProbPair& args, int n, hipStream_t st) {
     switch (variant) {
-        case 1: return launch_cfg<128, 256, 2, 2, 2, EPI, OUT_F32>(args, n, st);
-        case 2: return launch_cfg<256, 128, 2, 2, 2, EPI, OUT_F32>(args, n, st);
         case 4: return launch_cfg<256, 256, 2, 4, 2, EPI, OUT_F32>(args, n, st);
         default: return launch_cfg<128, 128, 2, 2, 2, EPI, OUT_F32>(args, n, st);
     }
@@ -307,6 +320,11 @@ int gemm_bf16_grouped(const GemmBf16Problem* probs, int n, int out_is_f32, int e
         d.A = q.A; d.Wp = q.Wp; d.out = q.out; d.ldc = q.ldc; d.M = q.M; d.N = q.N; d.K = q.K;
         d.epi = EpiDev{q.ea.bias, q.ea.gate, q.ea.resid, q.ea.table, q.ea.gate_ld, q.ea.rows_per_batch > 0 ? q.ea.rows_per_batch : 1};
         if (epi == EPI_BIAS_ROWADD) d.epi.gate_ld = q.N;
+        if (epi == EPI_QKV_NORM) {
+            if (q.N % 192 || !q.ea.gate || !q.ea.resid || (reinterpret_cast<uintptr_t>(q.ea.gate) & 15) || (reinterpret_cast<uintptr_t>(q.ea.resid) & 15))
+                return fail(SD3_ERR_INVALID_ARG, "gemm_bf16: the fused qk-norm needs N = 3C with C a multiple of 64 and two aligned weight vectors");
+            d.epi.gate_ld = q.N / 3;
+        }
         if (q.M > max_M) max_M = q.M;
     }
     if (m == 0) return SD3_OK;
@@ -319,6 +337,7 @@ int gemm_bf16_grouped(const GemmBf16Problem* probs, int n, int out_is_f32, int e
         case EPI_BIAS_SILU: SD3_GEMM_BF16_LAUNCH(EPI_BIAS_SILU);
         case EPI_GATE_RESID: SD3_GEMM_BF16_LAUNCH(EPI_GATE_RESID);
         case EPI_BIAS_ROWADD: SD3_GEMM_BF16_LAUNCH(EPI_BIAS_ROWADD);
+        case EPI_QKV_NORM: SD3_GEMM_BF16_LAUNCH(EPI_QKV_NORM);
         default: return fail(SD3_ERR_INVALID_ARG, "gemm_bf16: unknown epilogue %d", epi);
     }
 #undef SD3_GEMM_BF16_LAUNCH
