@@ -70,6 +70,9 @@ def main():
     ap.add_argument("--precision", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-events", action="store_true", help="do not record per-kernel events during the timed steps")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run one plain 1 GiB copy kernel (sd3::copy_rows_kernel), the known-size reference for scaling rocprofv3's "
+                         "FETCH_SIZE / WRITE_SIZE counters")
     a = ap.parse_args()
     if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on ONE GPU (no collectives, no sharding); use --gpus 1", file=sys.stderr)
@@ -102,6 +105,11 @@ def main():
     timesteps = torch.rand((B,), device=dev, generator=g) * 1000
     out = torch.empty_like(latent)
 
+    if a.copy_calibration:
+        src = torch.randn((1, 1 << 18, 1024), device=dev)  # 2^28 floats = 1 GiB read, 1 GiB written
+        M.concatenate_along_tokens(src, torch.empty((1, 0, 1024), device=dev))
+        torch.cuda.synchronize()
+        del src
     den = M.Denoiser(P, cfg, a.precision)
     for _ in range(max(a.warmup, 1) if a.warmup else 0):
         den(pooled, captions, latent, timesteps, out=out)

@@ -71,14 +71,12 @@ struct Prob {
 };
 struct ProbPair {
     Prob p[2];
-    int tiles0;
+    int tiles0, tiles_total;
 };
 
+// One output tile: K loop + epilogue. `wg` is the tile's position in the XCD-aware order of its problem.
 template <int BM, int BN, int WM, int WN, int STAGES, int EPI, bool OUT_F32>
-__global__ void __launch_bounds__(WM* WN * 64) gemm_bf16_kernel(const ProbPair args) {
-    const int which = (int)blockIdx.x >= args.tiles0 ? 1 : 0;
-    const int wg = (int)blockIdx.x - (which ? args.tiles0 : 0);
-    const Prob& pr = args.p[which];
+__device__ __forceinline__ void gemm_tile(const Prob& pr, const int wg, char* smem) {
     const bf16_t* __restrict__ A = pr.A;
     const bf16_t* __restrict__ Wp = pr.Wp;
     void* __restrict__ out_ = pr.out;
@@ -90,7 +88,6 @@ __global__ void __launch_bounds__(WM* WN * 64) gemm_bf16_kernel(const ProbPair a
     constexpr int LA = BM * 8 / NT, LB = BN * 8 / NT;        // 16-byte chunks per thread per tile
     static_assert(BM * 8 % NT == 0 && BN * 8 % NT == 0, "tile rows must divide evenly over the threads");
     static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0, "wavefront tiles are made of 32x32 blocks");
-    extern __shared__ __attribute__((aligned(1024))) char smem[];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WN, wn = wave % WN;
@@ -210,15 +207,22 @@ __global__ void __launch_bounds__(WM* WN * 64) gemm_bf16_kernel(const ProbPair a
         for (int j = 0; j < TN; j++)
 #pragma unroll
             for (int r = 0; r < 16; r++) slab[(8 * (r >> 2) + 4 * lk + (r & 3)) * EP + j * 32 + l32] = acc[i][j][r];
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        // LDS operations of one wavefront execute in program order, so the reads below see the writes above without a
+        // fence (a fence would also make the wavefront wait for its outstanding global stores on every pass)
         __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        // all rows of the slab are read into registers of their own before the first store is issued: a store keeps its data
+        // registers busy until it has left, so reusing one register set per row would put a full store round trip between rows
+        constexpr int NP = 32 / RPI;
+        float4 vals[NP];
 #pragma unroll
-        for (int p = 0; p < 32 / RPI; p++) {
+        for (int p = 0; p < NP; p++) vals[p] = *reinterpret_cast<const float4*>(&slab[(p * RPI + e_row) * EP + e_col]);
+        float4 res[NP];
+#pragma unroll
+        for (int p = 0; p < NP; p++) {
             const int row = p * RPI + e_row;
             const int m = m_blk + wm * (BM / WM) + i * 32 + row;
             if (m < M && nvalid > 0) {
-                const float4 a4 = *reinterpret_cast<const float4*>(&slab[row * EP + e_col]);
+                const float4 a4 = vals[p];
                 float v[4] = {a4.x + bias4[0], a4.y + bias4[1], a4.z + bias4[2], a4.w + bias4[3]};
                 const long long idx = (long long)m * ldc + n0;
                 if (EPI == EPI_BIAS_GELU) {
@@ -245,21 +249,32 @@ __global__ void __launch_bounds__(WM* WN * 64) gemm_bf16_kernel(const ProbPair a
                     for (int c = 0; c < 4; c++)
                         if (c < nvalid) v[c] += t[c];
                 }
-                if (EPI == EPI_QKV_NORM) {
-                    // the 16 lanes that hold this row's 64 columns are one head of one token (modules.cpp:192-198, fused)
-                    static_assert(EPI != EPI_QKV_NORM || WNC == 64, "the fused qk-norm needs one head per wavefront slab");
-                    const int third = (n_blk + wn * WNC) / epi.gate_ld;  // 0 = q, 1 = k, 2 = v (wavefront-uniform)
+                if constexpr (EPI == EPI_QKV_NORM && WNC % 64 == 0) {
+                    // 16 consecutive lanes hold 64 consecutive columns of this row = one head of one token (modules.cpp:192-198, fused)
+                    const int third = n0 / epi.gate_ld;  // 0 = q, 1 = k, 2 = v (uniform over the 16 lanes: C is a multiple of 64)
                     if (third < 2) {
-                        float ss = (v[0] * v[0] + v[1] * v[1]) + (v[2] * v[2] + v[3] * v[3]);
+                        // explicit fused multiply-adds: left to the compiler, each unrolled copy of this code may pick a different
+                        // product to fuse, and a row's result would depend on where in the tile it sits
+                        float ss = fmaf(v[3], v[3], fmaf(v[2], v[2], fmaf(v[1], v[1], v[0] * v[0])));
                         ss += __shfl_xor(ss, 1, 64);
                         ss += __shfl_xor(ss, 2, 64);
                         ss += __shfl_xor(ss, 4, 64);
                         ss += __shfl_xor(ss, 8, 64);
                         const float inv = 1.0f / sqrtf(1e-6f + ss * (1.0f / 64.0f));
-                        const float4 w4 = *reinterpret_cast<const float4*>((third == 0 ? epi.gate : epi.resid) + e_col);
-                        v[0] *= inv * w4.x; v[1] *= inv * w4.y; v[2] *= inv * w4.z; v[3] *= inv * w4.w;
+                        const float4 w4 = *reinterpret_cast<const float4*>((third == 0 ? epi.gate : epi.resid) + (n0 & 63));
+                        v[0] = (v[0] * inv) * w4.x; v[1] = (v[1] * inv) * w4.y; v[2] = (v[2] * inv) * w4.z; v[3] = (v[3] * inv) * w4.w;
                     }
                 }
+                res[p] = make_float4(v[0], v[1], v[2], v[3]);
+            }
+        }
+        // ... and all stores of the slab leave back to back
+#pragma unroll
+        for (int p = 0; p < NP; p++) {
+            const int m = m_blk + wm * (BM / WM) + i * 32 + p * RPI + e_row;
+            if (m < M && nvalid > 0) {
+                const long long idx = (long long)m * ldc + n0;
+                const float v[4] = {res[p].x, res[p].y, res[p].z, res[p].w};
                 if (vec_ok) {
                     if (OUT_F32) *reinterpret_cast<float4*>(outf + idx) = make_float4(v[0], v[1], v[2], v[3]);
                     else *reinterpret_cast<uint2*>(outh + idx) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
@@ -277,6 +292,19 @@ __global__ void __launch_bounds__(WM* WN * 64) gemm_bf16_kernel(const ProbPair a
     }
 }
 
+// Persistent kernel: one workgroup per compute unit walks over the tiles of up to two problems. The stores of a finished
+// tile drain while the next tile's K loop is already running, instead of holding the compute unit until they retire.
+// Workgroup g takes work items g, g + G, g + 2G ... (G = grid size, a multiple of 8), so it stays on its XCD's run of tiles.
+template <int BM, int BN, int WM, int WN, int STAGES, int EPI, bool OUT_F32>
+__global__ void __launch_bounds__(WM* WN * 64) gemm_bf16_kernel(const ProbPair args) {
+    extern __shared__ __attribute__((aligned(1024))) char smem[];
+    for (int w = blockIdx.x; w < args.tiles_total; w += gridDim.x) {
+        const int which = w >= args.tiles0 ? 1 : 0;
+        gemm_tile<BM, BN, WM, WN, STAGES, EPI, OUT_F32>(args.p[which], w - (which ? args.tiles0 : 0), smem);
+        __syncthreads();  // the staging slabs of this tile's epilogue alias the ring the next tile fills
+    }
+}
+
 template <int BM, int BN, int WM, int WN, int STAGES, int EPI, bool OUT_F32>
 int launch_cfg(ProbPair& args, int n, hipStream_t st) {
     auto kern = gemm_bf16_kernel<BM, BN, WM, WN, STAGES, EPI, OUT_F32>;
@@ -286,10 +314,23 @@ int launch_cfg(ProbPair& args, int n, hipStream_t st) {
         SD3_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, smem));
         attr_done = true;
     }
+    if (EPI == EPI_QKV_NORM && (BN / WN) % 64 != 0) return fail(SD3_ERR_UNSUPPORTED, "gemm_bf16: this tile shape cannot fuse the qk-norm");
     int tiles[2] = {0, 0};
     for (int i = 0; i < n; i++) tiles[i] = ((args.p[i].N + BN - 1) / BN) * ((args.p[i].M + BM - 1) / BM);
     args.tiles0 = tiles[0];
-    dim3 grid(tiles[0] + tiles[1]), block(WM * WN * 64);
+    args.tiles_total = tiles[0] + tiles[1];
+    // as many workgroups as can be resident at once (LDS allows one 256x256 or two 128x128 workgroups per compute unit), rounded
+    // down to a multiple of the 8 XCDs
+    static int resident = 0;
+    if (!resident) {
+        int dev = 0, cus = 0;
+        SD3_HIP_TRY(hipGetDevice(&dev));
+        SD3_HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+        const int per_cu = (160 * 1024) / smem > 0 ? (160 * 1024) / smem : 1;
+        resident = cus * (per_cu > 2 ? 2 : per_cu) / 8 * 8;
+        if (resident < 8) resident = 8;
+    }
+    dim3 grid(args.tiles_total < resident ? args.tiles_total : resident), block(WM * WN * 64);
     hipLaunchKernelGGL(kern, grid, block, smem, st, args);
     return launch_status("gemm_bf16");
 }
