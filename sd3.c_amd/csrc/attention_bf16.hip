@@ -25,8 +25,7 @@ constexpr int NW = 4;            // wavefronts per workgroup
 constexpr int QW = 64;           // queries per wavefront
 constexpr int BQ = NW * QW;      // queries per workgroup
 constexpr int BKV = 64;          // keys per tile
-constexpr int V_PITCH = 66;      // bf16 per V^T row (33 words: conflict-free transposing stores and 8-byte reads)
-constexpr int K_BYTES = BKV * 128, V_BYTES = HS * V_PITCH * 2, STAGE_BYTES = K_BYTES + V_BYTES;
+constexpr int K_BYTES = BKV * 128, V_BYTES = BKV * 128, STAGE_BYTES = K_BYTES + V_BYTES;
 constexpr int O_PITCH = 72;      // bf16 per staged output row
 constexpr int SMEM_BYTES = (2 * STAGE_BYTES > NW * QW * O_PITCH * 2) ? 2 * STAGE_BYTES : NW * QW * O_PITCH * 2;
 
@@ -62,6 +61,20 @@ union Frag {
     uint4 u;
     bf16x8_t v;
 };
+
+// ds_read_b64_tr_b16 works on blocks of 16 lanes: lane i of a block receives, as element j (of 4 bf16), element i%4 of the
+// 8 bytes addressed by lane (i/4 + 4j) of the block. Issued as inline assembly: through the compiler's builtin every such
+// read is preceded by s_waitcnt vmcnt(0), which would serialise it behind the global->LDS loads of the next tile. The
+// compiler does not count these reads, so the results may only be used after lds_wait() below has named them.
+__device__ __forceinline__ uint2 lds_read_tr16_b64(uint32_t lds_byte_addr, int imm_offset) {
+    uint2 r;
+    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(r) : "v"(lds_byte_addr), "i"(imm_offset));
+    return r;
+}
+__device__ __forceinline__ void lds_wait(uint2 (&a)[8]) {
+    asm volatile("s_waitcnt lgkmcnt(0)"
+                 : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(a[4]), "+v"(a[5]), "+v"(a[6]), "+v"(a[7]));
+}
 
 // NORM: apply the per-head RMSNorm to q and k while loading them (K then goes through registers instead of the
 // direct global->LDS path). Without it q and k are taken as they are (already normalised by the QKV GEMM epilogue).
@@ -132,21 +145,29 @@ __global__ void __launch_bounds__(NW * 64, 2) flash_attn_bf16_kernel(SegDev s, f
         for (int j = 0; j < 2; j++)
 #pragma unroll
             for (int r = 0; r < 16; r++) oacc[i][j][r] = 0.f;
+    // Softmax reference point m_run per query (any value works as long as numerator and denominator use the same one) and
+    // this lane's share l_run of the row sum. m_run is kept representable in bf16 because the matrix unit subtracts it:
+    // S^T starts from ONES . NEGM with NEGM[k=0][query] = -m_run and zeros elsewhere.
     float m_run[2] = {-1e30f, -1e30f}, l_run[2] = {0.f, 0.f};
-    constexpr float TAU = 8.0f;
     const bf16x2_t ONES = {(__bf16)1.0f, (__bf16)1.0f};
+    Frag ones_f, negm_f[2];
+    ones_f.u = make_uint4(0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u);
+#pragma unroll
+    for (int qb = 0; qb < 2; qb++) negm_f[qb].u = make_uint4(lk == 0 ? (pack_bf16x2(1e30f, 0.f) & 0xffffu) : 0u, 0u, 0u, 0u);
+    // a partial row sum of 16 probabilities above this bound (or infinite: always so on the first tile) moves the reference
+    constexpr float L_BOUND = 1073741824.0f;  // 2^30
 
-    // ---- staging roles ----
+    // ---- staging: chunk q = i*256 + tid of a tile lands at LDS byte q*16 of the K (V) area: row q/8, physical 16-byte
+    //      chunk q%8. The logical chunk fetched into that slot is XOR-swizzled per row so that the fragment reads below
+    //      are conflict-free: K by swz(row) (16-byte reads down a column of rows), V by 2*(row%4) (the transposing read
+    //      touches 32 bytes in each of 4 consecutive rows). ----
     auto kv_row_ptr = [&](const bf16_t* const* base, int t) -> const bf16_t* {
         t = min(t, T - 1);  // rows beyond the sequence re-read the last row: finite values, masked out of the softmax below
         const int seg = (t < T0) ? 0 : 1;
         return base[seg] + ((long long)b * s.T[seg] + (seg ? t - T0 : t)) * s.ld_qkv[seg] + h * HS;
     };
-    // K: chunk q = i*256 + tid of the tile lands at LDS byte q*16 (row q/8, physical chunk q%8, logical chunk XOR-swizzled)
-    // V: thread = (key pair, d-chunk): rows 2*vp and 2*vp+1, d = 8*v_ch..+7; stored transposed, two keys per 32-bit word
-    const int v_pair = tid >> 3, v_ch = tid & 7;
-    uint4 rk[2], rv[2];
-    // Row pointers of this thread's two K chunks and two V rows. Inside a segment they advance by a constant per tile;
+    uint4 rk[2];
+    // Row pointers of this thread's two K chunks and two V chunks. Inside a segment they advance by a constant per tile;
     // they are recomputed from scratch only for the first tile, the tiles around the segment boundary and the last tile.
     const bf16_t* kp[2];
     const bf16_t* vp[2];
@@ -163,141 +184,178 @@ __global__ void __launch_bounds__(NW * 64, 2) flash_attn_bf16_kernel(SegDev s, f
         } else {
 #pragma unroll
             for (int i = 0; i < 2; i++) {
-                const int q = i * 256 + tid, row = q >> 3, lc = (q & 7) ^ swz(row);
-                kp[i] = kv_row_ptr(s.k, t0 + row) + lc * 8;
-                vp[i] = kv_row_ptr(s.v, t0 + 2 * v_pair + i) + v_ch * 8;
+                const int q = i * 256 + tid, row = q >> 3;
+                kp[i] = kv_row_ptr(s.k, t0 + row) + ((q & 7) ^ swz(row)) * 8;
+                vp[i] = kv_row_ptr(s.v, t0 + row) + ((q & 7) ^ (2 * (row & 3))) * 8;
             }
         }
 #pragma unroll
         for (int i = 0; i < 2; i++) {
             if (NORM) rk[i] = *reinterpret_cast<const uint4*>(kp[i]);
             else __builtin_amdgcn_global_load_lds((glb_ptr_t)kp[i], (lds_ptr_t)(ks_ + (i * 256 + wave * 64) * 16), 16, 0, 0);
-            rv[i] = *reinterpret_cast<const uint4*>(vp[i]);
+            __builtin_amdgcn_global_load_lds((glb_ptr_t)vp[i], (lds_ptr_t)(ks_ + K_BYTES + (i * 256 + wave * 64) * 16), 16, 0, 0);
         }
     };
-    auto store_tile = [&](int t0, int stage) {
+    auto store_k_normed = [&](int t0, int stage) {  // NORM only: K rows pass through registers to be normalised
         char* ks_ = smem + stage * STAGE_BYTES;
-        if (NORM) {
 #pragma unroll
-            for (int i = 0; i < 2; i++) {
-                const int q = i * 256 + tid, row = q >> 3, lc = (q & 7) ^ swz(row);
-                const float* w = s.rms_k[(min(t0 + row, T - 1) < T0) ? 0 : 1];
-                uint4 u = rk[i];
-                if (w) {
-                    float f[8];
-                    unpack8(u, f);
-                    float ss = 0.f;
+        for (int i = 0; i < 2; i++) {
+            const int q = i * 256 + tid, row = q >> 3, lc = (q & 7) ^ swz(row);
+            const float* w = s.rms_k[(min(t0 + row, T - 1) < T0) ? 0 : 1];
+            uint4 u = rk[i];
+            if (w) {
+                float f[8];
+                unpack8(u, f);
+                float ss = 0.f;
 #pragma unroll
-                    for (int e = 0; e < 8; e++) ss += f[e] * f[e];
-                    ss += __shfl_xor(ss, 1, 64);  // the 8 chunks of a row sit in 8 consecutive lanes
-                    ss += __shfl_xor(ss, 2, 64);
-                    ss += __shfl_xor(ss, 4, 64);
-                    const float inv = 1.0f / sqrtf(eps + ss * (1.0f / HS));
+                for (int e = 0; e < 8; e++) ss += f[e] * f[e];
+                ss += __shfl_xor(ss, 1, 64);  // the 8 chunks of a row sit in 8 consecutive lanes
+                ss += __shfl_xor(ss, 2, 64);
+                ss += __shfl_xor(ss, 4, 64);
+                const float inv = 1.0f / sqrtf(eps + ss * (1.0f / HS));
 #pragma unroll
-                    for (int e = 0; e < 8; e++) f[e] *= inv * w[lc * 8 + e];
-                    u = pack8(f);
-                }
-                *reinterpret_cast<uint4*>(ks_ + q * 16) = u;
+                for (int e = 0; e < 8; e++) f[e] *= inv * w[lc * 8 + e];
+                u = pack8(f);
             }
-        }
-        // V^T[d][2*vp .. 2*vp+1] = (V[2vp][d], V[2vp+1][d])
-        const uint32_t a[4] = {rv[0].x, rv[0].y, rv[0].z, rv[0].w};
-        const uint32_t c[4] = {rv[1].x, rv[1].y, rv[1].z, rv[1].w};
-        uint32_t* vt32 = reinterpret_cast<uint32_t*>(ks_ + K_BYTES);
-#pragma unroll
-        for (int e = 0; e < 4; e++) {
-            vt32[((v_ch * 8 + 2 * e) * V_PITCH) / 2 + v_pair] = (a[e] & 0xffffu) | (c[e] << 16);            // d = 8*v_ch + 2e
-            vt32[((v_ch * 8 + 2 * e + 1) * V_PITCH) / 2 + v_pair] = (a[e] >> 16) | (c[e] & 0xffff0000u);    // d = 8*v_ch + 2e + 1
+            *reinterpret_cast<uint4*>(ks_ + q * 16) = u;
         }
     };
 
     const int nt = (T + BKV - 1) / BKV;
     issue_tile(0, 0);
-    store_tile(0, 0);
-    const int ksw = swz(l32);
+    if (NORM) store_k_normed(0, 0);
+    // Loop-invariant LDS byte offsets (relative to the stage) of this lane's operand fragments.
+    // K: the four 16-byte chunks (k-steps) of key row l32; 32-key blocks are a constant 32*128 bytes apart.
+    // V: with lane n of a 16-lane block pointing at V[key0 + n/4][d0 + 4*(n%4) ..], the transposing read leaves lane i
+    // with V[key0 + 0..3][d0 + i]: a column strip, i.e. half of a V^T operand row. The lane's block covers
+    // d0 = 32 db + 16 (lane/16 % 2) and key0 = (constant) + 4 lk.
+    int koff[4], voff[2];
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) koff[ks] = l32 * 128 + (((2 * ks + lk) ^ swz(l32)) * 16);
+    {
+        const int n = lane & 15, row = 4 * lk + (n >> 2);  // row % 4 == n / 4 for every constant added below (multiples of 8)
+#pragma unroll
+        for (int db = 0; db < 2; db++) {
+            const int chunk = db * 4 + 2 * ((lane >> 4) & 1) + ((n & 3) >> 1);
+            voff[db] = K_BYTES + row * 128 + ((chunk ^ (2 * (row & 3))) * 16) + 8 * (n & 1);
+        }
+    }
+    const uint32_t smem_addr = (uint32_t)(uintptr_t)(lds_ptr_t)smem;
+    const f32x16_t zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
     for (int t = 0; t < nt; t++) {
-        __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8));  // vmcnt(0): this thread's direct K loads of tile t have landed
+        __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8));  // vmcnt(0): this thread's direct loads of tile t have landed
         __syncthreads();  // tile t is complete in LDS, and every wavefront is done reading the other stage
         const bool more = t + 1 < nt;
         if (more) issue_tile((t + 1) * BKV, (t + 1) & 1);
         const char* ks_ = smem + (t & 1) * STAGE_BYTES;
-        const bf16_t* vt = reinterpret_cast<const bf16_t*>(ks_ + K_BYTES);
 
 #pragma unroll
         for (int kb = 0; kb < 2; kb++) {  // two 32-key halves of the tile
-            // ---- S^T = K . Q^T : one K fragment feeds both query blocks ----
-            f32x16_t sacc[2];
-            const f32x16_t zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int ks = 0; ks < 4; ks++) {
-                const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(ks_ + (kb * 32 + l32) * 128 + (((2 * ks + lk) ^ ksw) * 16));
-#pragma unroll
-                for (int qb = 0; qb < 2; qb++) sacc[qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[qb][ks].v, ks == 0 ? zero : sacc[qb], 0, 0, 0);
-            }
-            // register r is key  t*64 + 32 kb + 8 (r/4) + 4 lk + r%4
-            if (t == nt - 1) {
+            // register r of a score block is key  t*64 + 32 kb + 8 (r/4) + 4 lk + r%4
+            auto mask_tail = [&](f32x16_t (&sc)[2]) {
                 const int kbase = t * BKV + kb * 32 + 4 * lk;
 #pragma unroll
                 for (int r = 0; r < 16; r++)
                     if (kbase + 8 * (r >> 2) + (r & 3) >= T) {
-                        sacc[0][r] = -1e30f;
-                        sacc[1][r] = -1e30f;
+                        sc[0][r] = -1e30f;
+                        sc[1][r] = -1e30f;
                     }
-            }
-            // ---- online softmax per query block (base 2: log2(e)/8 is folded into q). The reference maximum m_run is only
-            //      raised when some score exceeds it by more than 2^TAU (probabilities then stay below 2^TAU, harmless in
-            //      fp32 / bf16), so the accumulator rescale runs on the first tile and hardly ever after that. ----
-            Frag pf[2][2];
-#pragma unroll
-            for (int qb = 0; qb < 2; qb++) {
-                float tmax = fmaxf(sacc[qb][0], sacc[qb][1]);
-#pragma unroll
-                for (int r = 2; r < 16; r += 2) tmax = fmaxf(tmax, fmaxf(sacc[qb][r], sacc[qb][r + 1]));
-                if (__any(tmax > m_run[qb] + TAU)) {
-                    // lanes l and l^32 hold the two key halves of the same query and feed the same accumulators: same reference
-                    const float m_new = fmaxf(m_run[qb], fmaxf(tmax, __shfl_xor(tmax, 32, 64)));
-                    const float alpha = __builtin_amdgcn_exp2f(m_run[qb] - m_new);
-                    m_run[qb] = m_new;
-                    l_run[qb] *= alpha;
-#pragma unroll
-                    for (int db = 0; db < 2; db++)
-#pragma unroll
-                        for (int r = 0; r < 16; r++) oacc[db][qb][r] *= alpha;
-                }
-                const float mref = m_run[qb];
-#pragma unroll
-                for (int r = 0; r < 16; r++) sacc[qb][r] = __builtin_amdgcn_exp2f(sacc[qb][r] - mref);
-                float ls0 = l_run[qb], ls1 = 0.f;
+            };
+            // probabilities of one query block -> bf16 P^T operands + this lane's sum of the rounded values
+            auto pack_probs = [&](const f32x16_t& pr, Frag (&pf)[2]) -> float {
+                float ls0 = 0.f, ls1 = 0.f;
 #pragma unroll
                 for (int j = 0; j < 2; j++) {
                     uint32_t w[4];
 #pragma unroll
                     for (int e = 0; e < 4; e++) {
-                        w[e] = pack_bf16x2(sacc[qb][8 * j + 2 * e], sacc[qb][8 * j + 2 * e + 1]);
-                        // row sum of the rounded probabilities, two per instruction
+                        w[e] = pack_bf16x2(pr[8 * j + 2 * e], pr[8 * j + 2 * e + 1]);
                         if (e & 1) ls1 = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, w[e]), ONES, ls1, false);
                         else ls0 = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, w[e]), ONES, ls0, false);
                     }
-                    pf[qb][j].u = make_uint4(w[0], w[1], w[2], w[3]);
+                    pf[j].u = make_uint4(w[0], w[1], w[2], w[3]);
                 }
-                l_run[qb] = ls0 + ls1;
+                return ls0 + ls1;
+            };
+
+            // ---- S^T - m = ONES . NEGM + K . Q^T : one K fragment feeds both query blocks ----
+            f32x16_t sacc[2];
+#pragma unroll
+            for (int qb = 0; qb < 2; qb++) sacc[qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ones_f.v, negm_f[qb].v, zero, 0, 0, 0);
+#pragma unroll
+            for (int ks = 0; ks < 4; ks++) {
+                const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(ks_ + koff[ks] + kb * 32 * 128);
+#pragma unroll
+                for (int qb = 0; qb < 2; qb++) sacc[qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[qb][ks].v, sacc[qb], 0, 0, 0);
             }
+            // V^T fragments of this half: [j][d block][keys 0-3 | keys 8-11 of the lane's 16-key step]; in flight during the softmax
+            uint2 vfr[8];
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+#pragma unroll
+                for (int db = 0; db < 2; db++)
+#pragma unroll
+                    for (int hi = 0; hi < 2; hi++)
+                        vfr[(j * 2 + db) * 2 + hi] = lds_read_tr16_b64(smem_addr + (t & 1) * STAGE_BYTES + voff[db], (kb * 32 + 16 * j + 8 * hi) * 128);
+            if (t == nt - 1) mask_tail(sacc);
+            // ---- probabilities (base 2: log2(e)/8 is folded into q) ----
+            Frag pf[2][2];
+            float inc[2];
+#pragma unroll
+            for (int qb = 0; qb < 2; qb++) {
+#pragma unroll
+                for (int r = 0; r < 16; r++) sacc[qb][r] = __builtin_amdgcn_exp2f(sacc[qb][r]);
+                inc[qb] = pack_probs(sacc[qb], pf[qb]);
+            }
+            if (__any(inc[0] + inc[1] > L_BOUND)) {
+                // Rare (always on the first tile, then only when scores outgrow the reference by 30 bits): recompute the raw
+                // scores, move the reference to the running maximum, rescale what has been accumulated, redo the probabilities.
+#pragma unroll
+                for (int ks = 0; ks < 4; ks++) {
+                    const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(ks_ + koff[ks] + kb * 32 * 128);
+#pragma unroll
+                    for (int qb = 0; qb < 2; qb++) sacc[qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[qb][ks].v, ks == 0 ? zero : sacc[qb], 0, 0, 0);
+                }
+                if (t == nt - 1) mask_tail(sacc);
+#pragma unroll
+                for (int qb = 0; qb < 2; qb++) {
+                    float tmax = fmaxf(sacc[qb][0], sacc[qb][1]);
+#pragma unroll
+                    for (int r = 2; r < 16; r += 2) tmax = fmaxf(tmax, fmaxf(sacc[qb][r], sacc[qb][r + 1]));
+                    // lanes l and l^32 hold the two key halves of the same query and feed the same accumulators: same reference
+                    const float m_new = fmaxf(m_run[qb], fmaxf(tmax, __shfl_xor(tmax, 32, 64)));
+                    const uint32_t negm_bits = pack_bf16x2(-m_new, 0.f) & 0xffffu;
+                    const float m_ref = -__uint_as_float(negm_bits << 16);
+                    const float alpha = __builtin_amdgcn_exp2f(m_run[qb] - m_ref);
+                    m_run[qb] = m_ref;
+                    negm_f[qb].u.x = lk == 0 ? negm_bits : 0u;
+                    l_run[qb] *= alpha;
+#pragma unroll
+                    for (int db = 0; db < 2; db++)
+#pragma unroll
+                        for (int r = 0; r < 16; r++) oacc[db][qb][r] *= alpha;
+#pragma unroll
+                    for (int r = 0; r < 16; r++) sacc[qb][r] = __builtin_amdgcn_exp2f(sacc[qb][r] - m_ref);
+                    inc[qb] = pack_probs(sacc[qb], pf[qb]);
+                }
+            }
+            l_run[0] += inc[0];
+            l_run[1] += inc[1];
             // ---- O^T += V^T . P^T ; step j contracts keys 32kb + 16j + {4lk..4lk+3, 8+4lk..8+4lk+3}; one V^T fragment feeds both query blocks ----
+            lds_wait(vfr);
 #pragma unroll
             for (int j = 0; j < 2; j++) {
-                const int key0 = kb * 32 + 16 * j + 4 * lk;
 #pragma unroll
                 for (int db = 0; db < 2; db++) {
-                    const uint32_t* row = reinterpret_cast<const uint32_t*>(&vt[(db * 32 + l32) * V_PITCH + key0]);
                     Frag vf;
-                    vf.u = make_uint4(row[0], row[1], row[4], row[5]);
+                    vf.u = make_uint4(vfr[(j * 2 + db) * 2].x, vfr[(j * 2 + db) * 2].y, vfr[(j * 2 + db) * 2 + 1].x, vfr[(j * 2 + db) * 2 + 1].y);
 #pragma unroll
                     for (int qb = 0; qb < 2; qb++) oacc[db][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf.v, pf[qb][j].v, oacc[db][qb], 0, 0, 0);
                 }
             }
         }
-        if (more) store_tile((t + 1) * BKV, (t + 1) & 1);
+        if (NORM && more) store_k_normed((t + 1) * BKV, (t + 1) & 1);
     }
 
     // ---- normalise; transpose through LDS (each wavefront its own 64-row region) so that rows leave as 16-byte stores ----
