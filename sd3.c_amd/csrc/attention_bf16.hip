@@ -27,7 +27,8 @@ constexpr int BQ = NW * QW;      // queries per workgroup
 constexpr int BKV = 64;          // keys per tile
 constexpr int K_BYTES = BKV * 128, V_BYTES = BKV * 128, STAGE_BYTES = K_BYTES + V_BYTES;
 constexpr int O_PITCH = 72;      // bf16 per staged output row
-constexpr int SMEM_BYTES = (2 * STAGE_BYTES > NW * QW * O_PITCH * 2) ? 2 * STAGE_BYTES : NW * QW * O_PITCH * 2;
+constexpr int NSTAGE = 3;
+constexpr int SMEM_BYTES = (NSTAGE * STAGE_BYTES > NW * QW * O_PITCH * 2) ? NSTAGE * STAGE_BYTES : NW * QW * O_PITCH * 2;
 
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 typedef const __attribute__((address_space(1))) void* glb_ptr_t;
@@ -146,15 +147,16 @@ __global__ void __launch_bounds__(NW * 64, 2) flash_attn_bf16_kernel(SegDev s, f
 #pragma unroll
             for (int r = 0; r < 16; r++) oacc[i][j][r] = 0.f;
     // Softmax reference point m_run per query (any value works as long as numerator and denominator use the same one) and
-    // this lane's share l_run of the row sum. m_run is kept representable in bf16 because the matrix unit subtracts it:
-    // S^T starts from ONES . NEGM with NEGM[k=0][query] = -m_run and zeros elsewhere.
-    float m_run[2] = {-1e30f, -1e30f}, l_run[2] = {0.f, 0.f};
+    // this lane's share l_run of the row sum. The matrix unit subtracts the reference and masks keys beyond the sequence:
+    // a score block starts from AUX . NEGM, where AUX[key][k=0] = 1, AUX[key][k=1] = (key beyond the sequence),
+    // NEGM[k=0][query] = -m_run (kept representable in bf16), NEGM[k=1][query] = -1e30 and everything else is zero.
+    float m_run[2] = {0.f, 0.f}, l_run[2] = {0.f, 0.f};
     const bf16x2_t ONES = {(__bf16)1.0f, (__bf16)1.0f};
-    Frag ones_f, negm_f[2];
-    ones_f.u = make_uint4(0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u);
+    const uint32_t NEG_BIG_HI = pack_bf16x2(0.f, -1e30f);  // bf16(-1e30) in the upper half
+    Frag negm_f[2];
 #pragma unroll
-    for (int qb = 0; qb < 2; qb++) negm_f[qb].u = make_uint4(lk == 0 ? (pack_bf16x2(1e30f, 0.f) & 0xffffu) : 0u, 0u, 0u, 0u);
-    // a partial row sum of 16 probabilities above this bound (or infinite: always so on the first tile) moves the reference
+    for (int qb = 0; qb < 2; qb++) negm_f[qb].u = make_uint4(lk == 0 ? NEG_BIG_HI : 0u, 0u, 0u, 0u);
+    // a partial row sum of 16 probabilities above this bound (or infinite) moves the reference
     constexpr float L_BOUND = 1073741824.0f;  // 2^30
 
     // ---- staging: chunk q = i*256 + tid of a tile lands at LDS byte q*16 of the K (V) area: row q/8, physical 16-byte
@@ -162,7 +164,7 @@ __global__ void __launch_bounds__(NW * 64, 2) flash_attn_bf16_kernel(SegDev s, f
     //      are conflict-free: K by swz(row) (16-byte reads down a column of rows), V by 2*(row%4) (the transposing read
     //      touches 32 bytes in each of 4 consecutive rows). ----
     auto kv_row_ptr = [&](const bf16_t* const* base, int t) -> const bf16_t* {
-        t = min(t, T - 1);  // rows beyond the sequence re-read the last row: finite values, masked out of the softmax below
+        t = min(t, T - 1);  // rows beyond the sequence re-read the last row: finite values, masked out of the softmax
         const int seg = (t < T0) ? 0 : 1;
         return base[seg] + ((long long)b * s.T[seg] + (seg ? t - T0 : t)) * s.ld_qkv[seg] + h * HS;
     };
@@ -171,8 +173,8 @@ __global__ void __launch_bounds__(NW * 64, 2) flash_attn_bf16_kernel(SegDev s, f
     // they are recomputed from scratch only for the first tile, the tiles around the segment boundary and the last tile.
     const bf16_t* kp[2];
     const bf16_t* vp[2];
-    auto issue_tile = [&](int t0, int stage) {
-        char* ks_ = smem + stage * STAGE_BYTES;
+    auto issue_tile = [&](int t0, int stage_byte) {
+        char* ks_ = smem + stage_byte;
         const bool in0 = (t0 >= BKV) && (t0 + BKV <= T0), in1 = (t0 - BKV >= T0) && (t0 + BKV <= T);
         if (in0 || in1) {
             const long long step = (long long)BKV * s.ld_qkv[in1 ? 1 : 0];
@@ -196,8 +198,8 @@ __global__ void __launch_bounds__(NW * 64, 2) flash_attn_bf16_kernel(SegDev s, f
             __builtin_amdgcn_global_load_lds((glb_ptr_t)vp[i], (lds_ptr_t)(ks_ + K_BYTES + (i * 256 + wave * 64) * 16), 16, 0, 0);
         }
     };
-    auto store_k_normed = [&](int t0, int stage) {  // NORM only: K rows pass through registers to be normalised
-        char* ks_ = smem + stage * STAGE_BYTES;
+    auto store_k_normed = [&](int t0, int stage_byte) {  // NORM only: K rows pass through registers to be normalised
+        char* ks_ = smem + stage_byte;
 #pragma unroll
         for (int i = 0; i < 2; i++) {
             const int q = i * 256 + tid, row = q >> 3, lc = (q & 7) ^ swz(row);
@@ -221,9 +223,6 @@ __global__ void __launch_bounds__(NW * 64, 2) flash_attn_bf16_kernel(SegDev s, f
         }
     };
 
-    const int nt = (T + BKV - 1) / BKV;
-    issue_tile(0, 0);
-    if (NORM) store_k_normed(0, 0);
     // Loop-invariant LDS byte offsets (relative to the stage) of this lane's operand fragments.
     // K: the four 16-byte chunks (k-steps) of key row l32; 32-key blocks are a constant 32*128 bytes apart.
     // V: with lane n of a 16-lane block pointing at V[key0 + n/4][d0 + 4*(n%4) ..], the transposing read leaves lane i
@@ -243,120 +242,180 @@ __global__ void __launch_bounds__(NW * 64, 2) flash_attn_bf16_kernel(SegDev s, f
     const uint32_t smem_addr = (uint32_t)(uintptr_t)(lds_ptr_t)smem;
     const f32x16_t zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
-    for (int t = 0; t < nt; t++) {
-        __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8));  // vmcnt(0): this thread's direct loads of tile t have landed
-        __syncthreads();  // tile t is complete in LDS, and every wavefront is done reading the other stage
-        const bool more = t + 1 < nt;
-        if (more) issue_tile((t + 1) * BKV, (t + 1) & 1);
-        const char* ks_ = smem + (t & 1) * STAGE_BYTES;
+    // ---- the pipeline. The unit of work is (32 keys) x (32 queries): unit u = (tile t, key half kb, query block qb), in
+    //      that order. Step u of the pipeline issues, interleaved in one instruction stream,
+    //        matrix unit:  the scores of unit u+1  and  O^T += V^T . P^T of unit u-1
+    //        vector unit:  the probabilities (exp2, bf16 rounding, row sums) of unit u
+    //      so that neither unit waits for the other inside a wavefront. Tiles live in a ring of three LDS stages: the
+    //      loads of tile t+2 are issued right after the barrier that publishes tile t+1, at which point every wavefront
+    //      has finished its reads of tile t-1, whose stage they overwrite. ----
+    const int nt = (T + BKV - 1) / BKV;
+    f32x16_t sacc[2];   // sacc[qb]: scores of the unit of query block qb that is in the pipeline
+    Frag pf[2][2];      // pf[qb][j]: its probabilities as P^T operands
+    bf16x8_t kf[4];     // K fragments of the key half whose scores are being issued
+    uint2 vfr[8];       // V^T fragments of the key half whose PV products are being issued: [j][d block][keys 0-3 | 8-11 of the step]
+#pragma unroll
+    for (int i = 0; i < 8; i++) vfr[i] = make_uint2(0u, 0u);
+#pragma unroll
+    for (int qb = 0; qb < 2; qb++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) pf[qb][j].u = make_uint4(0u, 0u, 0u, 0u);
 
+    auto aux_frag = [&](int key_base) -> Frag {  // AUX rows for keys key_base + l32
+        Frag f;
+        f.u = make_uint4((key_base + l32 >= T) ? 0x3f803f80u : 0x00003f80u, 0u, 0u, 0u);
+        return f;
+    };
+    auto scores = [&](int qb, const Frag& aux) {
+        sacc[qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(aux.v, negm_f[qb].v, zero, 0, 0, 0);
 #pragma unroll
-        for (int kb = 0; kb < 2; kb++) {  // two 32-key halves of the tile
-            // register r of a score block is key  t*64 + 32 kb + 8 (r/4) + 4 lk + r%4
-            auto mask_tail = [&](f32x16_t (&sc)[2]) {
-                const int kbase = t * BKV + kb * 32 + 4 * lk;
+        for (int ks = 0; ks < 4; ks++) sacc[qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[ks], qf[qb][ks].v, sacc[qb], 0, 0, 0);
+    };
+    auto load_k = [&](int stage_byte, int kb) {
 #pragma unroll
-                for (int r = 0; r < 16; r++)
-                    if (kbase + 8 * (r >> 2) + (r & 3) >= T) {
-                        sc[0][r] = -1e30f;
-                        sc[1][r] = -1e30f;
-                    }
-            };
-            // probabilities of one query block -> bf16 P^T operands + this lane's sum of the rounded values
-            auto pack_probs = [&](const f32x16_t& pr, Frag (&pf)[2]) -> float {
-                float ls0 = 0.f, ls1 = 0.f;
+        for (int ks = 0; ks < 4; ks++) kf[ks] = *reinterpret_cast<const bf16x8_t*>(smem + stage_byte + koff[ks] + kb * 32 * 128);
+    };
+    // probabilities of one unit -> bf16 P^T operands + this lane's sum of the rounded values
+    auto pack_probs = [&](const f32x16_t& pr, Frag (&out)[2]) -> float {
+        float ls0 = 0.f, ls1 = 0.f;
 #pragma unroll
-                for (int j = 0; j < 2; j++) {
-                    uint32_t w[4];
+        for (int j = 0; j < 2; j++) {
+            uint32_t w[4];
 #pragma unroll
-                    for (int e = 0; e < 4; e++) {
-                        w[e] = pack_bf16x2(pr[8 * j + 2 * e], pr[8 * j + 2 * e + 1]);
-                        if (e & 1) ls1 = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, w[e]), ONES, ls1, false);
-                        else ls0 = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, w[e]), ONES, ls0, false);
-                    }
-                    pf[j].u = make_uint4(w[0], w[1], w[2], w[3]);
-                }
-                return ls0 + ls1;
-            };
-
-            // ---- S^T - m = ONES . NEGM + K . Q^T : one K fragment feeds both query blocks ----
-            f32x16_t sacc[2];
-#pragma unroll
-            for (int qb = 0; qb < 2; qb++) sacc[qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ones_f.v, negm_f[qb].v, zero, 0, 0, 0);
-#pragma unroll
-            for (int ks = 0; ks < 4; ks++) {
-                const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(ks_ + koff[ks] + kb * 32 * 128);
-#pragma unroll
-                for (int qb = 0; qb < 2; qb++) sacc[qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[qb][ks].v, sacc[qb], 0, 0, 0);
+            for (int e = 0; e < 4; e++) {
+                w[e] = pack_bf16x2(pr[8 * j + 2 * e], pr[8 * j + 2 * e + 1]);
+                if (e & 1) ls1 = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, w[e]), ONES, ls1, false);
+                else ls0 = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, w[e]), ONES, ls0, false);
             }
-            // V^T fragments of this half: [j][d block][keys 0-3 | keys 8-11 of the lane's 16-key step]; in flight during the softmax
-            uint2 vfr[8];
-#pragma unroll
-            for (int j = 0; j < 2; j++)
-#pragma unroll
-                for (int db = 0; db < 2; db++)
-#pragma unroll
-                    for (int hi = 0; hi < 2; hi++)
-                        vfr[(j * 2 + db) * 2 + hi] = lds_read_tr16_b64(smem_addr + (t & 1) * STAGE_BYTES + voff[db], (kb * 32 + 16 * j + 8 * hi) * 128);
-            if (t == nt - 1) mask_tail(sacc);
-            // ---- probabilities (base 2: log2(e)/8 is folded into q) ----
-            Frag pf[2][2];
-            float inc[2];
-#pragma unroll
-            for (int qb = 0; qb < 2; qb++) {
-#pragma unroll
-                for (int r = 0; r < 16; r++) sacc[qb][r] = __builtin_amdgcn_exp2f(sacc[qb][r]);
-                inc[qb] = pack_probs(sacc[qb], pf[qb]);
-            }
-            if (__any(inc[0] + inc[1] > L_BOUND)) {
-                // Rare (always on the first tile, then only when scores outgrow the reference by 30 bits): recompute the raw
-                // scores, move the reference to the running maximum, rescale what has been accumulated, redo the probabilities.
-#pragma unroll
-                for (int ks = 0; ks < 4; ks++) {
-                    const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(ks_ + koff[ks] + kb * 32 * 128);
-#pragma unroll
-                    for (int qb = 0; qb < 2; qb++) sacc[qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[qb][ks].v, ks == 0 ? zero : sacc[qb], 0, 0, 0);
-                }
-                if (t == nt - 1) mask_tail(sacc);
-#pragma unroll
-                for (int qb = 0; qb < 2; qb++) {
-                    float tmax = fmaxf(sacc[qb][0], sacc[qb][1]);
-#pragma unroll
-                    for (int r = 2; r < 16; r += 2) tmax = fmaxf(tmax, fmaxf(sacc[qb][r], sacc[qb][r + 1]));
-                    // lanes l and l^32 hold the two key halves of the same query and feed the same accumulators: same reference
-                    const float m_new = fmaxf(m_run[qb], fmaxf(tmax, __shfl_xor(tmax, 32, 64)));
-                    const uint32_t negm_bits = pack_bf16x2(-m_new, 0.f) & 0xffffu;
-                    const float m_ref = -__uint_as_float(negm_bits << 16);
-                    const float alpha = __builtin_amdgcn_exp2f(m_run[qb] - m_ref);
-                    m_run[qb] = m_ref;
-                    negm_f[qb].u.x = lk == 0 ? negm_bits : 0u;
-                    l_run[qb] *= alpha;
-#pragma unroll
-                    for (int db = 0; db < 2; db++)
-#pragma unroll
-                        for (int r = 0; r < 16; r++) oacc[db][qb][r] *= alpha;
-#pragma unroll
-                    for (int r = 0; r < 16; r++) sacc[qb][r] = __builtin_amdgcn_exp2f(sacc[qb][r] - m_ref);
-                    inc[qb] = pack_probs(sacc[qb], pf[qb]);
-                }
-            }
-            l_run[0] += inc[0];
-            l_run[1] += inc[1];
-            // ---- O^T += V^T . P^T ; step j contracts keys 32kb + 16j + {4lk..4lk+3, 8+4lk..8+4lk+3}; one V^T fragment feeds both query blocks ----
-            lds_wait(vfr);
-#pragma unroll
-            for (int j = 0; j < 2; j++) {
-#pragma unroll
-                for (int db = 0; db < 2; db++) {
-                    Frag vf;
-                    vf.u = make_uint4(vfr[(j * 2 + db) * 2].x, vfr[(j * 2 + db) * 2].y, vfr[(j * 2 + db) * 2 + 1].x, vfr[(j * 2 + db) * 2 + 1].y);
-#pragma unroll
-                    for (int qb = 0; qb < 2; qb++) oacc[db][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf.v, pf[qb][j].v, oacc[db][qb], 0, 0, 0);
-                }
-            }
+            out[j].u = make_uint4(w[0], w[1], w[2], w[3]);
         }
-        if (NORM && more) store_k_normed((t + 1) * BKV, (t + 1) & 1);
+        return ls0 + ls1;
+    };
+    // O^T += V^T . P^T for query block qb; step j contracts keys 16j + {4lk..4lk+3, 8+4lk..8+4lk+3} of the key half in vfr
+    auto pv = [&](int qb) {
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int db = 0; db < 2; db++) {
+                Frag vf;
+                vf.u = make_uint4(vfr[(j * 2 + db) * 2].x, vfr[(j * 2 + db) * 2].y, vfr[(j * 2 + db) * 2 + 1].x, vfr[(j * 2 + db) * 2 + 1].y);
+                oacc[db][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf.v, pf[qb][j].v, oacc[db][qb], 0, 0, 0);
+            }
+    };
+    auto load_v = [&](int stage_byte, int kb) {
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int db = 0; db < 2; db++)
+#pragma unroll
+                for (int hi = 0; hi < 2; hi++)
+                    vfr[(j * 2 + db) * 2 + hi] = lds_read_tr16_b64(smem_addr + stage_byte + voff[db], (kb * 32 + 16 * j + 8 * hi) * 128);
+    };
+    // probabilities of the unit in sacc[qb] -> pf[qb]; returns this lane's row-sum increment
+    auto probs = [&](int qb) -> float {
+        f32x16_t pr;
+#pragma unroll
+        for (int r = 0; r < 16; r++) pr[r] = __builtin_amdgcn_exp2f(sacc[qb][r]);
+        return pack_probs(pr, pf[qb]);
+    };
+    // When the reference has to move (forced for the first units: they run with reference 0), the raw scores are
+    // recovered from the matrix unit's result, the reference goes to the running maximum, what was accumulated for this
+    // query block is rescaled and the probabilities are redone.
+    auto settle = [&](int qb, float inc, bool force) {
+        if (__any(inc > L_BOUND) || force) {
+            const float m_old = m_run[qb];
+            float tmax = fmaxf(sacc[qb][0], sacc[qb][1]);
+#pragma unroll
+            for (int r = 2; r < 16; r += 2) tmax = fmaxf(tmax, fmaxf(sacc[qb][r], sacc[qb][r + 1]));
+            // lanes l and l^32 hold the two key halves of the same query and feed the same accumulators: same reference
+            const float m_new = fmaxf(m_old, m_old + fmaxf(tmax, __shfl_xor(tmax, 32, 64)));
+            const uint32_t negm_bits = pack_bf16x2(-m_new, 0.f) & 0xffffu;
+            const float m_ref = -__uint_as_float(negm_bits << 16);
+            const float alpha = __builtin_amdgcn_exp2f(m_old - m_ref);
+            m_run[qb] = m_ref;
+            negm_f[qb].u.x = lk == 0 ? (negm_bits | NEG_BIG_HI) : 0u;
+            l_run[qb] *= alpha;
+#pragma unroll
+            for (int db = 0; db < 2; db++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) oacc[db][qb][r] *= alpha;
+            f32x16_t pr;
+#pragma unroll
+            for (int r = 0; r < 16; r++) pr[r] = __builtin_amdgcn_exp2f(sacc[qb][r] + (m_old - m_ref));
+            inc = pack_probs(pr, pf[qb]);
+        }
+        l_run[qb] += inc;
+    };
+    // one matrix instruction, then a few vector instructions, nine times: the mix of one pipeline step
+    auto interleave = [&]() {
+#pragma unroll
+        for (int i = 0; i < 9; i++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+        }
+    };
+
+    // prologue: tiles 0 and 1 on their way, tile 0 visible, scores of the first unit issued
+    issue_tile(0, 0);
+    if (NORM) store_k_normed(0, 0);
+    if (nt > 1) {
+        issue_tile(BKV, STAGE_BYTES);
+        __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8) | 4);  // vmcnt(4): all but the four loads of tile 1
+    } else {
+        __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8));
     }
+    __syncthreads();
+    load_k(0, 0);
+    scores(0, aux_frag(0));
+    int st_cur = 0, st_nxt = STAGE_BYTES, st_ld = 2 * STAGE_BYTES;  // stages of tiles t, t+1, t+2
+
+    for (int t = 0; t < nt; t++) {
+        const bool more = t + 1 < nt;
+        const Frag aux0 = aux_frag(t * BKV), aux1 = aux_frag(t * BKV + 32), auxn = aux_frag(t * BKV + BKV);
+        float inc;
+        // ---- step (t, 0, 0): scores of (t,0,1); PV of (t-1,1,1); then fetch K of half 1 and V of half 0 ----
+        scores(1, aux0);
+        load_k(st_cur, 1);
+        inc = probs(0);
+        pv(1);
+        load_v(st_cur, 0);
+        interleave();
+        settle(0, inc, t == 0);
+        // ---- step (t, 0, 1): scores of (t,1,0); PV of (t,0,0) ----
+        scores(0, aux1);
+        inc = probs(1);
+        lds_wait(vfr);
+        pv(0);
+        interleave();
+        settle(1, inc, t == 0);
+        // ---- step (t, 1, 0): tile t+1 becomes visible and tile t+2 sets off; scores of (t,1,1); PV of (t,0,1);
+        //      then fetch K of half 0 of tile t+1 and V of half 1 ----
+        if (more) {
+            if (NORM) store_k_normed((t + 1) * BKV, st_nxt);
+            __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8));  // vmcnt(0): this thread's loads of tile t+1 have landed
+            __syncthreads();
+            if (t + 2 < nt) issue_tile((t + 2) * BKV, st_ld);
+        }
+        scores(1, aux1);
+        load_k(st_nxt, 0);  // past the last tile: stale or unwritten LDS, feeding scores that are never used
+        inc = probs(0);
+        pv(1);
+        load_v(st_cur, 1);
+        interleave();
+        settle(0, inc, false);
+        // ---- step (t, 1, 1): scores of (t+1,0,0); PV of (t,1,0) ----
+        scores(0, auxn);
+        inc = probs(1);
+        lds_wait(vfr);
+        pv(0);
+        interleave();
+        settle(1, inc, false);
+        const int tmp = st_cur;
+        st_cur = st_nxt;
+        st_nxt = st_ld;
+        st_ld = tmp;
+    }
+    pv(1);  // PV of the last unit
 
     // ---- normalise; transpose through LDS (each wavefront its own 64-row region) so that rows leave as 16-byte stores ----
     __syncthreads();
