@@ -9,6 +9,8 @@
 // XOR-swizzled by a key of the row, which makes both the linear LDS fill and the 16-byte MFMA operand reads conflict-free.
 #include "common.hpp"
 
+#include <type_traits>
+
 namespace sd3 {
 namespace {
 
@@ -89,7 +91,8 @@ __device__ __forceinline__ void gemm_tile(const Prob& pr, const int wg, char* sm
     static_assert(BM * 8 % NT == 0 && BN * 8 % NT == 0, "tile rows must divide evenly over the threads");
     static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0, "wavefront tiles are made of 32x32 blocks");
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: LDS destinations of the direct loads are then scalar
     const int wm = wave / WN, wn = wave % WN;
     const int l32 = lane & 31, lk = lane >> 5;
     int tile_m, tile_n;
@@ -128,55 +131,79 @@ __device__ __forceinline__ void gemm_tile(const Prob& pr, const int wg, char* sm
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
+    static_assert(STAGES == 2, "the K loop below is written for a ring of two stages");
     const int nkt = K / BK;
-#pragma unroll
-    for (int s = 0; s < STAGES - 1; s++)
-        if (s < nkt) issue_tile(s, s);
 
     // operand addresses inside a stage: row*128 + ((2*ks + lk) ^ sw)*16 with sw = swz(row) = swz(l32) (block offsets are multiples of 16)
     const int sw = swz(l32);
     const int a_off = (wm * (BM / WM) + l32) * 128, b_off = A_BYTES + (wn * (BN / WN) + l32) * 128;
+    // operand fragments of k-step ks live in buffer ks&1; those of step ks+1 are fetched from LDS while the matrix cores work on step ks
+    bf16x8_t a[2][TM], b[2][TN];
+    auto fetch = [&](const char* st, int ks, int buf) {
+        const int ch = ((2 * ks + lk) ^ sw) * 16;
+#pragma unroll
+        for (int i = 0; i < TM; i++) a[buf][i] = *reinterpret_cast<const bf16x8_t*>(st + a_off + i * 32 * 128 + ch);
+#pragma unroll
+        for (int j = 0; j < TN; j++) b[buf][j] = *reinterpret_cast<const bf16x8_t*>(st + b_off + j * 32 * 128 + ch);
+    };
 
-    for (int kt = 0; kt < nkt; kt++) {
-        // tile kt has landed once at most (STAGES-2) newer tiles of this thread are still in flight
-        if (kt + STAGES - 1 <= nkt) wait_vmcnt<(STAGES - 2) * (LA + LB)>();
-        else wait_vmcnt<0>();
-        __syncthreads();  // everyone's part of tile kt is in LDS, and everyone is done reading the buffer refilled next
-        if (kt + STAGES - 1 < nkt) issue_tile(kt + STAGES - 1, (kt + STAGES - 1) % STAGES);
-        const char* st = smem + (kt % STAGES) * STAGE_BYTES;
-        // operand fragments of step ks+1 are fetched from LDS while the matrix cores work on step ks
-        bf16x8_t a[2][TM], b[2][TN];
-        auto fetch = [&](int ks, int buf) {
-            const int ch = ((2 * ks + lk) ^ sw) * 16;
-#pragma unroll
-            for (int i = 0; i < TM; i++) a[buf][i] = *reinterpret_cast<const bf16x8_t*>(st + a_off + i * 32 * 128 + ch);
-#pragma unroll
-            for (int j = 0; j < TN; j++) b[buf][j] = *reinterpret_cast<const bf16x8_t*>(st + b_off + j * 32 * 128 + ch);
-        };
-        fetch(0, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, TM + TN, 0);
-#pragma unroll
-        for (int ks = 0; ks < BK / 16; ks++) {
-            if (ks + 1 < BK / 16) fetch(ks + 1, (ks + 1) & 1);
+    issue_tile(0, 0);
+    wait_vmcnt<0>();
+    __syncthreads();  // tile 0 is in LDS
+    if (nkt > 1) issue_tile(1, 1);
+    fetch(smem, 0, 0);
+    __builtin_amdgcn_sched_group_barrier(0x100, TM + TN, 0);
+
+    constexpr int KS = BK / 16;
+    // One K tile. The workgroup barrier sits in front of the LAST k-step of a tile, not behind it: by then every fragment
+    // of tile kt is in registers (or on its way: waited for), so its buffer can be handed to the loads of tile kt+2, and the
+    // loads' issue and the first fragment reads of tile kt+1 are interleaved with the matrix instructions of that last
+    // step. With the barrier between tiles instead, the matrix pipeline drains at every tile boundary while all
+    // wavefronts of the compute unit wait for the barrier, issue their loads and wait for their first LDS reads.
+    auto k_tile = [&](const int kt, auto has_next_tag) {
+        constexpr bool HAS_NEXT = decltype(has_next_tag)::value;
+        const char* st = smem + (kt & 1) * STAGE_BYTES;
+        auto mfmas = [&](int buf) {
 #pragma unroll
             for (int i = 0; i < TM; i++)
 #pragma unroll
-                for (int j = 0; j < TN; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[ks & 1][i], b[ks & 1][j], acc[i][j], 0, 0, 0);
-            // scheduling pattern for this step: one LDS fragment read of the next step behind each of the first matrix
-            // instructions, so that LDS latency is covered by matrix work instead of a wait in front of every group
-            if (ks + 1 < BK / 16) {
+                for (int j = 0; j < TN; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[buf][i], b[buf][j], acc[i][j], 0, 0, 0);
+        };
+        // scheduling pattern of a step: behind each of the first matrix instructions one LDS fragment read of the next step
+        // (and, in the last step, one direct global->LDS load of the tile after next), so that their issue and latency are
+        // covered by matrix work
 #pragma unroll
-                for (int x = 0; x < TM + TN; x++) {
-                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
-                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // 1 DS read
-                }
-                __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - (TM + TN), 0);
-            } else {
-                __builtin_amdgcn_sched_group_barrier(0x008, TM * TN, 0);
+        for (int ks = 0; ks + 1 < KS; ks++) {
+            fetch(st, ks + 1, (ks + 1) & 1);
+            mfmas(ks & 1);
+#pragma unroll
+            for (int x = 0; x < TM + TN; x++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // 1 DS read
+            }
+            __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - (TM + TN), 0);
+        }
+        if (HAS_NEXT) {
+            __builtin_amdgcn_s_waitcnt(7 << 4);  // vmcnt(0): this thread's loads of tile kt+1 have landed; lgkmcnt(0): its reads of tile kt are done
+            __syncthreads();
+            issue_tile(min(kt + 2, nkt - 1), kt & 1);  // past the end: the last tile once more, into a buffer nobody reads again
+            fetch(smem + ((kt + 1) & 1) * STAGE_BYTES, 0, 0);
+        }
+        mfmas((KS - 1) & 1);
+        if (HAS_NEXT) {
+            constexpr int NLOADS = LA + LB, NM = TM * TN;
+            constexpr int LPS = (NLOADS + NM - 1) / NM;   // loads per slot
+            static_assert(TM + TN <= NM, "more fragment reads than matrix instructions to hide them behind");
+#pragma unroll
+            for (int x = 0; x < NM; x++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                              // 1 MFMA
+                if (x < TM + TN) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);              // 1 DS read
+                if (x * LPS < NLOADS) __builtin_amdgcn_sched_group_barrier(0x020, LPS, 0);       // VMEM reads
             }
         }
-    }
+    };
+    for (int kt = 0; kt + 1 < nkt; kt++) k_tile(kt, std::true_type{});
+    k_tile(nkt - 1, std::false_type{});
 
     // ---- epilogue. The MFMA C layout (lane = column, register r = row 8*(r/4) + 4*(lane/32) + r%4) would give 2- or
     // 4-byte scattered stores; each wavefront instead transposes one 32-row slab at a time through its private LDS
