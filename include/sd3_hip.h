@@ -155,6 +155,10 @@ int sd3_pack_weight_bf16(const float* W, void* wpacked, int K, int N, void* stre
 int sd3_gemm_bf16(const void* A, const void* wpacked, const float* bias, void* out, int M, int N, int K, int epilogue, void* stream);
 /* fp32 -> bf16 (round to nearest even) */
 int sd3_cast_f32_to_bf16(const float* in, void* out, long long n, void* stream);
+/* Tuning hook with no counterpart in the reference: forces the output tile of the bf16 GEMM for every later call in this
+ * process. tile = 0: chosen per call from the problem sizes (the default); 128: 128x128 tiles, two workgroups per compute
+ * unit; 256: 256x256 tiles, one workgroup per compute unit. Results do not depend on the choice. */
+int sd3_gemm_bf16_force_tile(int tile);
 
 #ifdef __cplusplus
 }

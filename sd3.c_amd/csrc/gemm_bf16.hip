@@ -332,6 +332,20 @@ __global__ void __launch_bounds__(WM* WN * 64) gemm_bf16_kernel(const ProbPair a
     }
 }
 
+// compute units of the current device (0 after a failed query, which has set the error message)
+int compute_units() {
+    static int cus = 0;
+    if (!cus) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
+            fail(SD3_ERR_HIP, "gemm_bf16: cannot query the number of compute units");
+            return 0;
+        }
+        cus = n;
+    }
+    return cus;
+}
+
 template <int BM, int BN, int WM, int WN, int STAGES, int EPI, bool OUT_F32>
 int launch_cfg(ProbPair& args, int n, hipStream_t st) {
     auto kern = gemm_bf16_kernel<BM, BN, WM, WN, STAGES, EPI, OUT_F32>;
@@ -348,15 +362,10 @@ int launch_cfg(ProbPair& args, int n, hipStream_t st) {
     args.tiles_total = tiles[0] + tiles[1];
     // as many workgroups as can be resident at once (LDS allows one 256x256 or two 128x128 workgroups per compute unit), rounded
     // down to a multiple of the 8 XCDs
-    static int resident = 0;
-    if (!resident) {
-        int dev = 0, cus = 0;
-        SD3_HIP_TRY(hipGetDevice(&dev));
-        SD3_HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-        const int per_cu = (160 * 1024) / smem > 0 ? (160 * 1024) / smem : 1;
-        resident = cus * (per_cu > 2 ? 2 : per_cu) / 8 * 8;
-        if (resident < 8) resident = 8;
-    }
+    const int cus = compute_units();
+    if (cus <= 0) return SD3_ERR_HIP;
+    constexpr int per_cu = (160 * 1024) / smem > 1 ? 2 : 1;
+    const int resident = (cus * per_cu / 8 * 8) > 8 ? (cus * per_cu / 8 * 8) : 8;
     dim3 grid(args.tiles_total < resident ? args.tiles_total : resident), block(WM * WN * 64);
     hipLaunchKernelGGL(kern, grid, block, smem, st, args);
     return launch_status("gemm_bf16");
@@ -372,7 +381,7 @@ int launch_epi(int variant, ProbPair& args, int n, hipStream_t st) {
 
 }  // namespace
 
-int g_gemm_bf16_variant = -1;  // -1: choose by shape; >= 0: tuning knob (tile shape), see launch_epi
+int g_gemm_bf16_variant = -1;  // -1: choose by shape; 0 / 4: forced 128x128 / 256x256 tiles (sd3_gemm_bf16_force_tile)
 
 int gemm_bf16_grouped(const GemmBf16Problem* probs, int n, int out_is_f32, int epi, hipStream_t st) {
     if (n < 1 || n > 2) return fail(SD3_ERR_INVALID_ARG, "gemm_bf16_grouped: 1 or 2 problems (got %d)", n);
@@ -396,19 +405,41 @@ int gemm_bf16_grouped(const GemmBf16Problem* probs, int n, int out_is_f32, int e
         if (q.M > max_M) max_M = q.M;
     }
     if (m == 0) return SD3_OK;
-    // tile shape: 256x256 (8 wavefronts) for large problems, 128x128 (4 wavefronts) when there are few rows
-    const int v = g_gemm_bf16_variant >= 0 ? g_gemm_bf16_variant : (max_M >= 1024 ? 4 : 0);
-#define SD3_GEMM_BF16_LAUNCH(E) return out_is_f32 ? launch_epi<E, true>(v, args, m, st) : launch_epi<E, false>(v, args, m, st)
-    switch (epi) {
-        case EPI_BIAS: SD3_GEMM_BF16_LAUNCH(EPI_BIAS);
-        case EPI_BIAS_GELU: SD3_GEMM_BF16_LAUNCH(EPI_BIAS_GELU);
-        case EPI_BIAS_SILU: SD3_GEMM_BF16_LAUNCH(EPI_BIAS_SILU);
-        case EPI_GATE_RESID: SD3_GEMM_BF16_LAUNCH(EPI_GATE_RESID);
-        case EPI_BIAS_ROWADD: SD3_GEMM_BF16_LAUNCH(EPI_BIAS_ROWADD);
-        case EPI_QKV_NORM: SD3_GEMM_BF16_LAUNCH(EPI_QKV_NORM);
-        default: return fail(SD3_ERR_INVALID_ARG, "gemm_bf16: unknown epilogue %d", epi);
-    }
+    auto launch = [&](ProbPair& pp, int count, int v) -> int {
+#define SD3_GEMM_BF16_LAUNCH(E) return out_is_f32 ? launch_epi<E, true>(v, pp, count, st) : launch_epi<E, false>(v, pp, count, st)
+        switch (epi) {
+            case EPI_BIAS: SD3_GEMM_BF16_LAUNCH(EPI_BIAS);
+            case EPI_BIAS_GELU: SD3_GEMM_BF16_LAUNCH(EPI_BIAS_GELU);
+            case EPI_BIAS_SILU: SD3_GEMM_BF16_LAUNCH(EPI_BIAS_SILU);
+            case EPI_GATE_RESID: SD3_GEMM_BF16_LAUNCH(EPI_GATE_RESID);
+            case EPI_BIAS_ROWADD: SD3_GEMM_BF16_LAUNCH(EPI_BIAS_ROWADD);
+            case EPI_QKV_NORM: SD3_GEMM_BF16_LAUNCH(EPI_QKV_NORM);
+            default: return fail(SD3_ERR_INVALID_ARG, "gemm_bf16: unknown epilogue %d", epi);
+        }
 #undef SD3_GEMM_BF16_LAUNCH
+    };
+    if (g_gemm_bf16_variant >= 0) return launch(args, m, g_gemm_bf16_variant);
+    // tile shape: 256x256 (8 wavefronts, one workgroup per compute unit) for large problems, 128x128 (4 wavefronts, two
+    // workgroups per compute unit) when there are few rows
+    const int v = max_M >= 1024 ? 4 : 0;
+    if (m == 2 && v == 4) {
+        // A persistent launch takes ceil(tiles / compute units) rounds of tile time. When the small problem's tiles push the
+        // pair into one more round than the large problem needs alone, the small one goes first in a launch of its own with
+        // small tiles (a short single round) instead of costing a whole round of large tiles.
+        const int cus = compute_units();
+        if (cus <= 0) return SD3_ERR_HIP;
+        auto tiles256 = [](const Prob& q) { return ((q.M + 255) / 256) * ((q.N + 255) / 256); };
+        const int big = args.p[0].M >= args.p[1].M ? 0 : 1, small = 1 - big;
+        const int t_big = tiles256(args.p[big]), t_both = t_big + tiles256(args.p[small]);
+        if (args.p[small].M < 1024 && (t_both + cus - 1) / cus > (t_big + cus - 1) / cus) {
+            ProbPair one{};
+            one.p[0] = args.p[small];
+            SD3_TRY(launch(one, 1, 0));
+            one.p[0] = args.p[big];
+            return launch(one, 1, 4);
+        }
+    }
+    return launch(args, m, v);
 }
 
 int gemm_bf16(const bf16_t* A, const bf16_t* Wp, void* out, int out_is_f32, int ldc, int M, int N, int K, int epi, const GemmEpilogueArgs& ea,
@@ -419,7 +450,8 @@ int gemm_bf16(const bf16_t* A, const bf16_t* Wp, void* out, int out_is_f32, int 
 
 }  // namespace sd3
 
-extern "C" int sd3_dev_set_gemm_variant(int v) {
-    sd3::g_gemm_bf16_variant = v;
-    return 0;
+extern "C" int sd3_gemm_bf16_force_tile(int tile) {
+    if (tile != 0 && tile != 128 && tile != 256) return sd3::fail(SD3_ERR_INVALID_ARG, "sd3_gemm_bf16_force_tile: tile must be 0, 128 or 256 (got %d)", tile);
+    sd3::g_gemm_bf16_variant = tile == 0 ? -1 : (tile == 256 ? 4 : 0);
+    return SD3_OK;
 }

@@ -50,6 +50,7 @@ SIGNATURES = {
     "sd3_pack_weight_bf16": [vp, vp, ci, ci, vp],
     "sd3_gemm_bf16": [vp, vp, vp, vp, ci, ci, ci, ci, vp],
     "sd3_cast_f32_to_bf16": [vp, vp, cll, vp],
+    "sd3_gemm_bf16_force_tile": [ci],
 }
 
 

@@ -84,6 +84,50 @@ def test_gemm_bf16(Mr, N, K, epi):
     assert rel_l2(host(out), host(ref)) <= 5e-3  # bf16 rounding of the output is 2^-9 relative
 
 
+@pytest.mark.parametrize("Mr,N,K,epi", [(2304, 1536, 1536, 1), (300, 320, 6144, 0)])
+def test_gemm_bf16_result_does_not_depend_on_tile_shape(Mr, N, K, epi):
+    """Every output element is accumulated over K in the same order whatever tile it falls into: bit-identical results."""
+    g = torch.Generator(device="cuda").manual_seed(K + N)
+    A = torch.randn((Mr, K), device="cuda", generator=g).bfloat16()
+    Wp = (0.05 * torch.randn((N, K), device="cuda", generator=g)).bfloat16()
+    bias = torch.randn(N, device="cuda", generator=g)
+    outs = []
+    try:
+        for tile in (128, 256, 0):
+            L.call("sd3_gemm_bf16_force_tile", tile)
+            out = torch.zeros((Mr, N), device="cuda", dtype=torch.bfloat16)
+            L.call("sd3_gemm_bf16", A.data_ptr(), Wp.data_ptr(), bias.data_ptr(), out.data_ptr(), Mr, N, K, epi, None)
+            outs.append(out)
+    finally:
+        L.call("sd3_gemm_bf16_force_tile", 0)
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
+    with pytest.raises(L.Sd3Error):
+        L.call("sd3_gemm_bf16_force_tile", 64)
+
+
+def test_flash_attention_bf16_late_maximum_moves_the_reference():
+    """The last keys score about 40 bits above everything before them, so the reference point of the online softmax has
+    to move long after the first tile (the rescale path) and the early keys must fade out without overflow. Large scores
+    amplify the rounding of the pre-scaled bf16 query operand, so the comparison is against fp32 arithmetic on that same
+    rounded operand (q * log2(e)/8 in bf16), which is what the kernel documents it multiplies."""
+    B, T1, NH, HS = 1, 300, 2, 64
+    C = NH * HS
+    g = torch.Generator(device="cuda").manual_seed(11)
+    qkv = torch.randn((B * T1, 3 * C), device="cuda", generator=g)
+    qkv[-5:, C:2 * C] *= 12.0      # the last five keys dominate
+    qkv = qkv.bfloat16()
+    out = torch.zeros((B * T1, C), device="cuda", dtype=torch.bfloat16)
+    L.call("sd3_flash_attention_bf16", qkv.data_ptr(), None, out.data_ptr(), None, None, None, None, None, B, T1, 0, NH, HS, None)
+    q, k, v = qkv.float().view(B, T1, 3, NH, HS).unbind(2)
+    q2 = (q * (1.4426950408889634 / 8.0)).bfloat16().float()
+    s2 = torch.einsum("bqhd,bkhd->bhqk", q2, k)
+    assert float(s2.max()) > 40.0  # base-2 exponents: far beyond the 2^30 head-room of a fixed reference
+    p = torch.exp2(s2 - s2.max(-1, keepdim=True).values)
+    ref = torch.einsum("bhqk,bkhd->bqhd", p / p.sum(-1, keepdim=True), v).reshape(B * T1, C)
+    assert torch.isfinite(out.float()).all()
+    assert float((out.float() - ref).abs().max()) <= 0.05
+
+
 def test_cast_rounds_to_nearest_even():
     x = torch.randn(100000, device="cuda") * 100
     x[:4] = torch.tensor([0.0, -0.0, float("inf"), 1.00390625])  # the last one is exactly halfway between two bf16 values
