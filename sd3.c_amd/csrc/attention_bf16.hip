@@ -66,15 +66,19 @@ union Frag {
 // ds_read_b64_tr_b16 works on blocks of 16 lanes: lane i of a block receives, as element j (of 4 bf16), element i%4 of the
 // 8 bytes addressed by lane (i/4 + 4j) of the block. Issued as inline assembly: through the compiler's builtin every such
 // read is preceded by s_waitcnt vmcnt(0), which would serialise it behind the global->LDS loads of the next tile. The
-// compiler does not count these reads, so the results may only be used after lds_wait() below has named them.
+// compiler does not count these reads, so the results may only be used after one of the waits below has named them.
 __device__ __forceinline__ uint2 lds_read_tr16_b64(uint32_t lds_byte_addr, int imm_offset) {
     uint2 r;
     asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(r) : "v"(lds_byte_addr), "i"(imm_offset));
     return r;
 }
-__device__ __forceinline__ void lds_wait(uint2 (&a)[8]) {
-    asm volatile("s_waitcnt lgkmcnt(0)"
-                 : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(a[4]), "+v"(a[5]), "+v"(a[6]), "+v"(a[7]));
+// The transposing reads are issued in two groups of four (first vfr[0..3], then vfr[4..7]). LDS operations complete in order, so
+// once at most four are outstanding the first group has landed whatever else the compiler has put in between.
+__device__ __forceinline__ void lds_wait_first4(uint2 (&a)[8]) {
+    asm volatile("s_waitcnt lgkmcnt(4)" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]));
+}
+__device__ __forceinline__ void lds_wait_last4(uint2 (&a)[8]) {
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a[4]), "+v"(a[5]), "+v"(a[6]), "+v"(a[7]));
 }
 
 // NORM: apply the per-head RMSNorm to q and k while loading them (K then goes through registers instead of the
@@ -82,7 +86,8 @@ __device__ __forceinline__ void lds_wait(uint2 (&a)[8]) {
 template <bool NORM>
 __global__ void __launch_bounds__(NW * 64, 2) flash_attn_bf16_kernel(SegDev s, float q_scale /* log2(e)/sqrt(64) */, float eps) {
     __shared__ __attribute__((aligned(1024))) char smem[SMEM_BYTES];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: LDS destinations of the direct loads are then scalar
     const int l32 = lane & 31, lk = lane >> 5;
     const int T0 = s.T[0], T = s.T[0] + s.T[1];
     const int Tq0 = s.Tq[0], TQ = s.Tq[0] + s.Tq[1];
@@ -173,8 +178,9 @@ __global__ void __launch_bounds__(NW * 64, 2) flash_attn_bf16_kernel(SegDev s, f
     // they are recomputed from scratch only for the first tile, the tiles around the segment boundary and the last tile.
     const bf16_t* kp[2];
     const bf16_t* vp[2];
-    auto issue_tile = [&](int t0, int stage_byte) {
-        char* ks_ = smem + stage_byte;
+    // advance() moves the four row pointers to the tile that starts at key t0 (branches; kept out of the pipeline steps),
+    // fetch_tile() issues the loads through them (straight-line; interleaved with a step's matrix instructions)
+    auto advance = [&](int t0) {
         const bool in0 = (t0 >= BKV) && (t0 + BKV <= T0), in1 = (t0 - BKV >= T0) && (t0 + BKV <= T);
         if (in0 || in1) {
             const long long step = (long long)BKV * s.ld_qkv[in1 ? 1 : 0];
@@ -191,6 +197,9 @@ __global__ void __launch_bounds__(NW * 64, 2) flash_attn_bf16_kernel(SegDev s, f
                 vp[i] = kv_row_ptr(s.v, t0 + row) + ((q & 7) ^ (2 * (row & 3))) * 8;
             }
         }
+    };
+    auto fetch_tile = [&](int stage_byte) {
+        char* ks_ = smem + stage_byte;
 #pragma unroll
         for (int i = 0; i < 2; i++) {
             if (NORM) rk[i] = *reinterpret_cast<const uint4*>(kp[i]);
@@ -291,25 +300,22 @@ __global__ void __launch_bounds__(NW * 64, 2) flash_attn_bf16_kernel(SegDev s, f
         }
         return ls0 + ls1;
     };
-    // O^T += V^T . P^T for query block qb; step j contracts keys 16j + {4lk..4lk+3, 8+4lk..8+4lk+3} of the key half in vfr
-    auto pv = [&](int qb) {
+    // O^T += V^T . P^T for query block qb, half j of it: contracts keys 16j + {4lk..4lk+3, 8+4lk..8+4lk+3} of the key half in vfr
+    auto pv = [&](int qb, int j) {
 #pragma unroll
-        for (int j = 0; j < 2; j++)
-#pragma unroll
-            for (int db = 0; db < 2; db++) {
-                Frag vf;
-                vf.u = make_uint4(vfr[(j * 2 + db) * 2].x, vfr[(j * 2 + db) * 2].y, vfr[(j * 2 + db) * 2 + 1].x, vfr[(j * 2 + db) * 2 + 1].y);
-                oacc[db][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf.v, pf[qb][j].v, oacc[db][qb], 0, 0, 0);
-            }
+        for (int db = 0; db < 2; db++) {
+            Frag vf;
+            vf.u = make_uint4(vfr[(j * 2 + db) * 2].x, vfr[(j * 2 + db) * 2].y, vfr[(j * 2 + db) * 2 + 1].x, vfr[(j * 2 + db) * 2 + 1].y);
+            oacc[db][qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf.v, pf[qb][j].v, oacc[db][qb], 0, 0, 0);
+        }
     };
-    auto load_v = [&](int stage_byte, int kb) {
+    // the V^T fragments of half j of key half kb: issued as soon as the products that used the previous contents are issued
+    auto load_v = [&](int stage_byte, int kb, int j) {
 #pragma unroll
-        for (int j = 0; j < 2; j++)
+        for (int db = 0; db < 2; db++)
 #pragma unroll
-            for (int db = 0; db < 2; db++)
-#pragma unroll
-                for (int hi = 0; hi < 2; hi++)
-                    vfr[(j * 2 + db) * 2 + hi] = lds_read_tr16_b64(smem_addr + stage_byte + voff[db], (kb * 32 + 16 * j + 8 * hi) * 128);
+            for (int hi = 0; hi < 2; hi++)
+                vfr[(j * 2 + db) * 2 + hi] = lds_read_tr16_b64(smem_addr + stage_byte + voff[db], (kb * 32 + 16 * j + 8 * hi) * 128);
     };
     // probabilities of the unit in sacc[qb] -> pf[qb]; returns this lane's row-sum increment
     auto probs = [&](int qb) -> float {
@@ -356,10 +362,12 @@ __global__ void __launch_bounds__(NW * 64, 2) flash_attn_bf16_kernel(SegDev s, f
     };
 
     // prologue: tiles 0 and 1 on their way, tile 0 visible, scores of the first unit issued
-    issue_tile(0, 0);
+    advance(0);
+    fetch_tile(0);
     if (NORM) store_k_normed(0, 0);
     if (nt > 1) {
-        issue_tile(BKV, STAGE_BYTES);
+        advance(BKV);
+        fetch_tile(STAGE_BYTES);
         __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8) | 4);  // vmcnt(4): all but the four loads of tile 1
     } else {
         __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8));
@@ -370,44 +378,51 @@ __global__ void __launch_bounds__(NW * 64, 2) flash_attn_bf16_kernel(SegDev s, f
     int st_cur = 0, st_nxt = STAGE_BYTES, st_ld = 2 * STAGE_BYTES;  // stages of tiles t, t+1, t+2
 
     for (int t = 0; t < nt; t++) {
-        const bool more = t + 1 < nt;
-        const Frag aux0 = aux_frag(t * BKV), aux1 = aux_frag(t * BKV + 32), auxn = aux_frag(t * BKV + BKV);
         float inc;
-        // ---- step (t, 0, 0): scores of (t,0,1); PV of (t-1,1,1); then fetch K of half 1 and V of half 0 ----
-        scores(1, aux0);
+        // ---- step (t, 0, 0): PV of (t-1,1,1), each half followed by the fetch of V of key half 0 into the registers it
+        //      frees; scores of (t,0,1); then fetch K of half 1 ----
+        pv(1, 0);
+        load_v(st_cur, 0, 0);
+        scores(1, aux_frag(t * BKV));
         load_k(st_cur, 1);
         inc = probs(0);
-        pv(1);
-        load_v(st_cur, 0);
+        pv(1, 1);
+        load_v(st_cur, 0, 1);
         interleave();
         settle(0, inc, t == 0);
-        // ---- step (t, 0, 1): scores of (t,1,0); PV of (t,0,0) ----
-        scores(0, aux1);
+        // ---- step (t, 0, 1): PV of (t,0,0); scores of (t,1,0) ----
+        lds_wait_first4(vfr);
+        pv(0, 0);
+        scores(0, aux_frag(t * BKV + 32));
         inc = probs(1);
-        lds_wait(vfr);
-        pv(0);
+        lds_wait_last4(vfr);
+        pv(0, 1);
         interleave();
         settle(1, inc, t == 0);
-        // ---- step (t, 1, 0): tile t+1 becomes visible and tile t+2 sets off; scores of (t,1,1); PV of (t,0,1);
-        //      then fetch K of half 0 of tile t+1 and V of half 1 ----
-        if (more) {
-            if (NORM) store_k_normed((t + 1) * BKV, st_nxt);
-            __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8));  // vmcnt(0): this thread's loads of tile t+1 have landed
-            __syncthreads();
-            if (t + 2 < nt) issue_tile((t + 2) * BKV, st_ld);
-        }
-        scores(1, aux1);
-        load_k(st_nxt, 0);  // past the last tile: stale or unwritten LDS, feeding scores that are never used
+        // ---- step (t, 1, 0): tile t+1 becomes visible and the loads of tile t+2 set off (past the end: the last tile once
+        //      more, into a stage nobody reads again); PV of (t,0,1) and fetch of V of key half 1; scores of (t,1,1); then
+        //      fetch K of half 0 of tile t+1 (past the last tile: stale LDS, feeding scores that are never used) ----
+        if (NORM && t + 1 < nt) store_k_normed((t + 1) * BKV, st_nxt);
+        __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8));  // vmcnt(0): this thread's loads of tile t+1 have landed
+        __syncthreads();  // (also in the last tile: the stage the redundant loads go to must not be in use by a slower wavefront)
+        if (t + 2 < nt) advance((t + 2) * BKV);
+        fetch_tile(st_ld);
+        pv(1, 0);
+        load_v(st_cur, 1, 0);
+        scores(1, aux_frag(t * BKV + 32));
+        load_k(st_nxt, 0);
         inc = probs(0);
-        pv(1);
-        load_v(st_cur, 1);
+        pv(1, 1);
+        load_v(st_cur, 1, 1);
         interleave();
         settle(0, inc, false);
-        // ---- step (t, 1, 1): scores of (t+1,0,0); PV of (t,1,0) ----
-        scores(0, auxn);
+        // ---- step (t, 1, 1): PV of (t,1,0); scores of (t+1,0,0) ----
+        lds_wait_first4(vfr);
+        pv(0, 0);
+        scores(0, aux_frag(t * BKV + BKV));
         inc = probs(1);
-        lds_wait(vfr);
-        pv(0);
+        lds_wait_last4(vfr);
+        pv(0, 1);
         interleave();
         settle(1, inc, false);
         const int tmp = st_cur;
@@ -415,7 +430,9 @@ __global__ void __launch_bounds__(NW * 64, 2) flash_attn_bf16_kernel(SegDev s, f
         st_nxt = st_ld;
         st_ld = tmp;
     }
-    pv(1);  // PV of the last unit
+    pv(1, 0);  // PV of the last unit
+    pv(1, 1);
+    __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8));  // the redundant loads issued past the last tile have landed before LDS is reused
 
     // ---- normalise; transpose through LDS (each wavefront its own 64-row region) so that rows leave as 16-byte stores ----
     __syncthreads();
