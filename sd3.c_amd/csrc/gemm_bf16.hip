@@ -228,8 +228,28 @@ __device__ __forceinline__ void gemm_tile(const Prob& pr, const int wg, char* sm
             if (c < nvalid) bias4[c] = epi.bias[n0 + c];
     // batch index of a row without a division per row: the tile starts in batch b0 and crosses a boundary every rpb rows
     const int rpb = epi.rows_per_batch, b0 = m_blk / rpb;
+    constexpr int NP = 32 / RPI;        // rows of a slab per lane
+    // gated layers: the residual rows of the NEXT slab are requested before the current slab goes through LDS, so that
+    // their latency is not paid once per slab with nothing else to do
+    constexpr bool PREFETCH_RESID = (EPI == EPI_GATE_RESID);
+    float4 rnext[PREFETCH_RESID ? NP : 1];
+    auto request_resid = [&](int i) {
+        if (PREFETCH_RESID && vec_ok)
+#pragma unroll
+            for (int p = 0; p < NP; p++) {
+                const int m = m_blk + wm * (BM / WM) + i * 32 + p * RPI + e_row;
+                if (m < M && nvalid > 0) rnext[p] = *reinterpret_cast<const float4*>(epi.resid + (long long)m * ldc + n0);
+            }
+    };
+    request_resid(0);
 #pragma unroll
     for (int i = 0; i < TM; i++) {
+        float4 rcur[PREFETCH_RESID ? NP : 1];
+        if (PREFETCH_RESID) {
+#pragma unroll
+            for (int p = 0; p < NP; p++) rcur[p] = rnext[p];
+            if (i + 1 < TM) request_resid(i + 1);
+        }
 #pragma unroll
         for (int j = 0; j < TN; j++)
 #pragma unroll
@@ -239,7 +259,6 @@ __device__ __forceinline__ void gemm_tile(const Prob& pr, const int wg, char* sm
         __builtin_amdgcn_wave_barrier();
         // all rows of the slab are read into registers of their own before the first store is issued: a store keeps its data
         // registers busy until it has left, so reusing one register set per row would put a full store round trip between rows
-        constexpr int NP = 32 / RPI;
         float4 vals[NP];
 #pragma unroll
         for (int p = 0; p < NP; p++) vals[p] = *reinterpret_cast<const float4*>(&slab[(p * RPI + e_row) * EP + e_col]);
@@ -263,7 +282,7 @@ __device__ __forceinline__ void gemm_tile(const Prob& pr, const int wg, char* sm
                     for (int nb = (b0 + 1) * rpb; nb <= m; nb += rpb) bi++;  // at most BM/rpb + 1 steps, 0 or 1 in practice
                     const float* g = epi.gate + (long long)bi * epi.gate_ld + n0;
                     if (vec_ok) {
-                        const float4 g4 = *reinterpret_cast<const float4*>(g), r4 = *reinterpret_cast<const float4*>(epi.resid + idx);
+                        const float4 g4 = *reinterpret_cast<const float4*>(g), r4 = rcur[PREFETCH_RESID ? p : 0];
                         v[0] = r4.x + g4.x * v[0]; v[1] = r4.y + g4.y * v[1]; v[2] = r4.z + g4.z * v[2]; v[3] = r4.w + g4.w * v[3];
                     } else {
 #pragma unroll
