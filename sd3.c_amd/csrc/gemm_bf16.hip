@@ -131,7 +131,7 @@ __device__ __forceinline__ void gemm_tile(const Prob& pr, const int wg, char* sm
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
-    static_assert(STAGES == 2, "the K loop below is written for a ring of two stages");
+    static_assert(STAGES >= 2 && (STAGES - 1) * (LA + LB) < 64, "ring depth: at least two stages, and the loads in flight must fit the 6-bit counter");
     const int nkt = K / BK;
 
     // operand addresses inside a stage: row*128 + ((2*ks + lk) ^ sw)*16 with sw = swz(row) = swz(l32) (block offsets are multiples of 16)
@@ -147,10 +147,15 @@ __device__ __forceinline__ void gemm_tile(const Prob& pr, const int wg, char* sm
         for (int j = 0; j < TN; j++) b[buf][j] = *reinterpret_cast<const bf16x8_t*>(st + b_off + j * 32 * 128 + ch);
     };
 
-    issue_tile(0, 0);
-    wait_vmcnt<0>();
-    __syncthreads();  // tile 0 is in LDS
-    if (nkt > 1) issue_tile(1, 1);
+    // Every stage is filled up front and exactly one tile is requested per K tile after that (past the end: the last tile
+    // once more, into a buffer nobody reads again), so "tile kt+1 has landed" is always "all but the newest STAGES-2 tiles".
+#pragma unroll
+    for (int s = 0; s < STAGES; s++) issue_tile(min(s, nkt - 1), s);
+    wait_vmcnt<(STAGES - 1) * (LA + LB)>();
+    // tile 0 is in LDS. A bare barrier between compiler fences: __syncthreads() would add a wait for ALL loads in flight
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
     fetch(smem, 0, 0);
     __builtin_amdgcn_sched_group_barrier(0x100, TM + TN, 0);
 
@@ -162,7 +167,7 @@ __device__ __forceinline__ void gemm_tile(const Prob& pr, const int wg, char* sm
     // wavefronts of the compute unit wait for the barrier, issue their loads and wait for their first LDS reads.
     auto k_tile = [&](const int kt, auto has_next_tag) {
         constexpr bool HAS_NEXT = decltype(has_next_tag)::value;
-        const char* st = smem + (kt & 1) * STAGE_BYTES;
+        const char* st = smem + (kt % STAGES) * STAGE_BYTES;
         auto mfmas = [&](int buf) {
 #pragma unroll
             for (int i = 0; i < TM; i++)
@@ -184,10 +189,14 @@ __device__ __forceinline__ void gemm_tile(const Prob& pr, const int wg, char* sm
             __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - (TM + TN), 0);
         }
         if (HAS_NEXT) {
-            __builtin_amdgcn_s_waitcnt(7 << 4);  // vmcnt(0): this thread's loads of tile kt+1 have landed; lgkmcnt(0): its reads of tile kt are done
-            __syncthreads();
-            issue_tile(min(kt + 2, nkt - 1), kt & 1);  // past the end: the last tile once more, into a buffer nobody reads again
-            fetch(smem + ((kt + 1) & 1) * STAGE_BYTES, 0, 0);
+            // this thread's loads of tile kt+1 have landed (vmcnt: all but the newest STAGES-2 tiles) and its reads of tile kt are done (lgkmcnt(0))
+            constexpr int INFLIGHT = (STAGES - 2) * (LA + LB);
+            __builtin_amdgcn_s_waitcnt((INFLIGHT & 15) | (7 << 4) | ((INFLIGHT >> 4) << 14));
+            asm volatile("" ::: "memory");  // (the barrier builtin alone does not keep the compiler from moving LDS reads across it)
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+            issue_tile(min(kt + STAGES, nkt - 1), kt % STAGES);
+            fetch(smem + ((kt + 1) % STAGES) * STAGE_BYTES, 0, 0);
         }
         mfmas((KS - 1) & 1);
         if (HAS_NEXT) {
@@ -394,13 +403,14 @@ template <int EPI, bool OUT_F32>
 int launch_epi(int variant, ProbPair& args, int n, hipStream_t st) {
     switch (variant) {
         case 4: return launch_cfg<256, 256, 2, 4, 2, EPI, OUT_F32>(args, n, st);
+        case 1: return launch_cfg<128, 128, 2, 2, 4, EPI, OUT_F32>(args, n, st);
         default: return launch_cfg<128, 128, 2, 2, 2, EPI, OUT_F32>(args, n, st);
     }
 }
 
 }  // namespace
 
-int g_gemm_bf16_variant = -1;  // -1: choose by shape; 0 / 4: forced 128x128 / 256x256 tiles (sd3_gemm_bf16_force_tile)
+int g_gemm_bf16_variant = -1;  // -1: choose by shape; 0 / 4: forced 128x128 / 256x256 tiles (sd3_gemm_bf16_force_tile); 1: 128x128 with a ring of four stages
 
 int gemm_bf16_grouped(const GemmBf16Problem* probs, int n, int out_is_f32, int epi, hipStream_t st) {
     if (n < 1 || n > 2) return fail(SD3_ERR_INVALID_ARG, "gemm_bf16_grouped: 1 or 2 problems (got %d)", n);
@@ -440,7 +450,16 @@ int gemm_bf16_grouped(const GemmBf16Problem* probs, int n, int out_is_f32, int e
     if (g_gemm_bf16_variant >= 0) return launch(args, m, g_gemm_bf16_variant);
     // tile shape: 256x256 (8 wavefronts, one workgroup per compute unit) for large problems, 128x128 (4 wavefronts, two
     // workgroups per compute unit) when there are few rows
-    const int v = max_M >= 1024 ? 4 : 0;
+    int v = max_M >= 1024 ? 4 : 0;
+    if (v == 0) {
+        // few rows and no more 128x128 tiles than compute units: one workgroup per unit, so LDS can hold a ring of four
+        // stages, which is what counts when the launch is a single short round bound by load latency
+        const int cus = compute_units();
+        if (cus <= 0) return SD3_ERR_HIP;
+        int tiles128 = 0;
+        for (int i = 0; i < m; i++) tiles128 += ((args.p[i].M + 127) / 128) * ((args.p[i].N + 127) / 128);
+        if (tiles128 <= cus) v = 1;
+    }
     if (m == 2 && v == 4) {
         // A persistent launch takes ceil(tiles / compute units) rounds of tile time. When the small problem's tiles push the
         // pair into one more round than the large problem needs alone, the small one goes first in a launch of its own with
@@ -453,7 +472,8 @@ int gemm_bf16_grouped(const GemmBf16Problem* probs, int n, int out_is_f32, int e
         if (args.p[small].M < 1024 && (t_both + cus - 1) / cus > (t_big + cus - 1) / cus) {
             ProbPair one{};
             one.p[0] = args.p[small];
-            SD3_TRY(launch(one, 1, 0));
+            const int small_tiles = ((one.p[0].M + 127) / 128) * ((one.p[0].N + 127) / 128);
+            SD3_TRY(launch(one, 1, small_tiles <= cus ? 1 : 0));
             one.p[0] = args.p[big];
             return launch(one, 1, 4);
         }
