@@ -54,6 +54,7 @@ struct sd3_ctx {
         hipEvent_t a, b;
         int cls;
         double work;
+        long long launches;
     };
     std::vector<ProfSample> prof;
     std::vector<hipEvent_t> event_pool;
@@ -131,7 +132,8 @@ struct ProfScope {
     hipEvent_t a = nullptr, b = nullptr;
     int cls;
     double work;
-    ProfScope(sd3_ctx* c, int cls_, double work_) : ctx(c), cls(cls_), work(work_) {
+    long long gemm_launches_before;  // one bracketed call may launch more than one GEMM kernel; the class counts kernels
+    ProfScope(sd3_ctx* c, int cls_, double work_) : ctx(c), cls(cls_), work(work_), gemm_launches_before(g_gemm_bf16_launches) {
         if (!ctx->prof_on) return;
         auto get = [&]() -> hipEvent_t {
             hipEvent_t e = nullptr;
@@ -151,7 +153,8 @@ struct ProfScope {
     ~ProfScope() {
         if (!a || !b) return;
         (void)hipEventRecord(b, ctx->stream);
-        ctx->prof.push_back({a, b, cls, work});
+        const long long kernels = g_gemm_bf16_launches - gemm_launches_before;
+        ctx->prof.push_back({a, b, cls, work, kernels > 1 ? kernels : 1});
     }
 };
 
@@ -692,7 +695,7 @@ int sd3_profile_end(sd3_ctx* ctx, double* ms, double* work, long long* launches)
         SD3_HIP_TRY(hipEventElapsedTime(&t, p.a, p.b));
         ms[p.cls] += t;
         work[p.cls] += p.work;
-        launches[p.cls] += 1;
+        launches[p.cls] += p.launches;
         ctx->event_pool.push_back(p.a);
         ctx->event_pool.push_back(p.b);
     }
