@@ -170,6 +170,7 @@ size_t block_workspace_bytes(const Dims& d, int prec) {
     auto act = [&](size_t n) { b.take<char>(n * es); };
     act(mc * d.C); act(mx * d.C); act(mx * d.C);           // c_hid, x_hid, x_hid2
     act(mc * 3 * d.C); act(mx * 3 * d.C);                  // c_qkv, x_qkv
+    if (d.dual) act(mx * 3 * d.C);                         // x_qkv2
     act(mc * d.C); act(mx * d.C);                          // c_att, x_att
     act(mc * d.E * d.C); act(mx * d.E * d.C);              // c_mlp, x_mlp
     b.take<float>((size_t)d.B * 6 * d.C); b.take<float>((size_t)d.B * 9 * d.C);  // ada_c, ada_x
@@ -209,7 +210,8 @@ int linear_pair(sd3_ctx* ctx, int prec, const LayerCall* calls, int n, int out_f
         }
         return SD3_OK;
     }
-    GemmBf16Problem probs[2];
+    GemmBf16Problem probs[3];
+    if (n > 3) return fail(SD3_ERR_INVALID_ARG, "linear_pair: at most three layers per group");
     int m = 0;
     double flop = 0;
     for (int i = 0; i < n; i++) {
@@ -271,6 +273,7 @@ int run_block(sd3_ctx* ctx, int prec, const float* y, float* c, float* x, const 
     void* x_hid2 = act((size_t)mx * C);
     void* c_qkv = act((size_t)mc * 3 * C);
     void* x_qkv = act((size_t)mx * 3 * C);
+    void* x_qkv2 = d.dual ? act((size_t)mx * 3 * C) : nullptr;  // q,k,v of the extra self-attention branch
     void* c_att = act((size_t)mc * C);
     void* x_att = act((size_t)mx * C);
     void* c_mlp = act((size_t)mc * d.E * C);
@@ -317,9 +320,13 @@ int run_block(sd3_ctx* ctx, int prec, const float* y, float* c, float* x, const 
         nx.gate = w.x_rms_q; nx.resid = w.x_rms_k;
         nc.gate = w.c_rms_q; nc.resid = w.c_rms_k;
         const bool fused_norm = bf && d.qk;
-        LayerCall qkv[2] = {{x_hid, w.x_qkv_w, w.x_qkv_b, x_qkv, 3 * C, mx, 3 * C, C, fused_norm ? nx : none},
+        GemmEpilogueArgs n2;
+        n2.gate = w.x2_rms_q; n2.resid = w.x2_rms_k;
+        // the dual branch's projection reads the other output of the same LayerNorm pass: same kind, same launch
+        LayerCall qkv[3] = {{x_hid, w.x_qkv_w, w.x_qkv_b, x_qkv, 3 * C, mx, 3 * C, C, fused_norm ? nx : none},
+                            {x_hid2, w.x2_qkv_w, w.x2_qkv_b, x_qkv2, 3 * C, d.dual ? mx : 0, 3 * C, C, fused_norm ? n2 : none},
                             {c_hid, w.c_qkv_w, w.c_qkv_b, c_qkv, 3 * C, mc, 3 * C, C, fused_norm ? nc : none}};
-        SD3_TRY(linear_pair(ctx, prec, qkv, 2, !bf, fused_norm ? EPI_QKV_NORM : EPI_BIAS));
+        SD3_TRY(linear_pair(ctx, prec, qkv, 3, !bf, fused_norm ? EPI_QKV_NORM : EPI_BIAS));
     }
 
     // ---- joint attention over [context ; latent] (modules.cpp:1427-1432); fp32 path: qk-norm in place first
@@ -349,16 +356,12 @@ int run_block(sd3_ctx* ctx, int prec, const float* y, float* c, float* x, const 
 
     // ---- extra self-attention over the latent tokens (modules.cpp:1440-1453, 1486)
     if (d.dual) {
-        GemmEpilogueArgs n2;
-        n2.gate = w.x2_rms_q; n2.resid = w.x2_rms_k;
-        SD3_TRY(linear_layer(ctx, prec, x_hid2, w.x2_qkv_w, w.x2_qkv_b, x_qkv, !bf, 3 * C, mx, 3 * C, C, (bf && d.qk) ? EPI_QKV_NORM : EPI_BIAS,
-                             (bf && d.qk) ? n2 : none));
         if (!bf && d.qk) {
-            SD3_TRY(rmsnorm_rows((float*)x_qkv, (float*)x_qkv, w.x2_rms_q, nullptr, 1e-6f, mx, d.NH, d.HS, 3 * C, 3 * C, st));
-            SD3_TRY(rmsnorm_rows((float*)seg_ptr(x_qkv, 1), (float*)seg_ptr(x_qkv, 1), w.x2_rms_k, nullptr, 1e-6f, mx, d.NH, d.HS, 3 * C, 3 * C, st));
+            SD3_TRY(rmsnorm_rows((float*)x_qkv2, (float*)x_qkv2, w.x2_rms_q, nullptr, 1e-6f, mx, d.NH, d.HS, 3 * C, 3 * C, st));
+            SD3_TRY(rmsnorm_rows((float*)seg_ptr(x_qkv2, 1), (float*)seg_ptr(x_qkv2, 1), w.x2_rms_k, nullptr, 1e-6f, mx, d.NH, d.HS, 3 * C, 3 * C, st));
         }
         AttnSegments a{};
-        a.q[0] = x_qkv; a.k[0] = seg_ptr(x_qkv, 1); a.v[0] = seg_ptr(x_qkv, 2); a.out[0] = x_att;
+        a.q[0] = x_qkv2; a.k[0] = seg_ptr(x_qkv2, 1); a.v[0] = seg_ptr(x_qkv2, 2); a.out[0] = x_att;
         a.ld_qkv[0] = a.ld_qkv[1] = 3 * C; a.ld_out[0] = a.ld_out[1] = C;
         a.T[0] = a.Tq[0] = Tx;
         SD3_TRY(attention(ctx, a, B, d.NH, d.HS, bf));

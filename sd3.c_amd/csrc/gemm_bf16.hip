@@ -62,8 +62,8 @@ constexpr int smem_bytes() {
     return ring > epi ? ring : epi;
 }
 
-// One launch covers up to two independent problems (the latent-stream and the context-stream layer of the same kind):
-// workgroups [0, tiles0) belong to problem 0, the rest to problem 1.
+// One launch covers up to three independent problems of the same kind (latent-stream, dual-branch and context-stream
+// layer): work items [0, end[0]) belong to problem 0, [end[0], end[1]) to problem 1, [end[1], end[2]) to problem 2.
 struct Prob {
     const bf16_t* A;
     const bf16_t* Wp;
@@ -71,9 +71,10 @@ struct Prob {
     int ldc, M, N, K;
     EpiDev epi;
 };
-struct ProbPair {
-    Prob p[2];
-    int tiles0, tiles_total;
+constexpr int MAX_PROBS = 3;
+struct ProbSet {
+    Prob p[MAX_PROBS];
+    int end[MAX_PROBS];  // running totals of tiles
 };
 
 // One output tile: K loop + epilogue. `wg` is the tile's position in the XCD-aware order of its problem.
@@ -351,11 +352,11 @@ __device__ __forceinline__ void gemm_tile(const Prob& pr, const int wg, char* sm
 // tile drain while the next tile's K loop is already running, instead of holding the compute unit until they retire.
 // Workgroup g takes work items g, g + G, g + 2G ... (G = grid size, a multiple of 8), so it stays on its XCD's run of tiles.
 template <int BM, int BN, int WM, int WN, int STAGES, int EPI, bool OUT_F32>
-__global__ void __launch_bounds__(WM* WN * 64) gemm_bf16_kernel(const ProbPair args) {
+__global__ void __launch_bounds__(WM* WN * 64) gemm_bf16_kernel(const ProbSet args) {
     extern __shared__ __attribute__((aligned(1024))) char smem[];
-    for (int w = blockIdx.x; w < args.tiles_total; w += gridDim.x) {
-        const int which = w >= args.tiles0 ? 1 : 0;
-        gemm_tile<BM, BN, WM, WN, STAGES, EPI, OUT_F32>(args.p[which], w - (which ? args.tiles0 : 0), smem);
+    for (int w = blockIdx.x; w < args.end[MAX_PROBS - 1]; w += gridDim.x) {
+        const int which = (w >= args.end[0]) + (w >= args.end[1]);
+        gemm_tile<BM, BN, WM, WN, STAGES, EPI, OUT_F32>(args.p[which], w - (which ? args.end[which - 1] : 0), smem);
         __syncthreads();  // the staging slabs of this tile's epilogue alias the ring the next tile fills
     }
 }
@@ -375,7 +376,7 @@ int compute_units() {
 }
 
 template <int BM, int BN, int WM, int WN, int STAGES, int EPI, bool OUT_F32>
-int launch_cfg(ProbPair& args, int n, hipStream_t st) {
+int launch_cfg(ProbSet& args, int n, hipStream_t st) {
     auto kern = gemm_bf16_kernel<BM, BN, WM, WN, STAGES, EPI, OUT_F32>;
     constexpr int smem = smem_bytes<BM, BN, WM, WN, STAGES>();
     static bool attr_done = false;  // raising the dynamic LDS limit is a per-function, per-process setting
@@ -384,24 +385,25 @@ int launch_cfg(ProbPair& args, int n, hipStream_t st) {
         attr_done = true;
     }
     if (EPI == EPI_QKV_NORM && (BN / WN) % 64 != 0) return fail(SD3_ERR_UNSUPPORTED, "gemm_bf16: this tile shape cannot fuse the qk-norm");
-    int tiles[2] = {0, 0};
-    for (int i = 0; i < n; i++) tiles[i] = ((args.p[i].N + BN - 1) / BN) * ((args.p[i].M + BM - 1) / BM);
-    args.tiles0 = tiles[0];
-    args.tiles_total = tiles[0] + tiles[1];
+    int total = 0;
+    for (int i = 0; i < MAX_PROBS; i++) {
+        if (i < n) total += ((args.p[i].N + BN - 1) / BN) * ((args.p[i].M + BM - 1) / BM);
+        args.end[i] = total;
+    }
     // as many workgroups as can be resident at once (LDS allows one 256x256 or two 128x128 workgroups per compute unit), rounded
     // down to a multiple of the 8 XCDs
     const int cus = compute_units();
     if (cus <= 0) return SD3_ERR_HIP;
     constexpr int per_cu = (160 * 1024) / smem > 1 ? 2 : 1;
     const int resident = (cus * per_cu / 8 * 8) > 8 ? (cus * per_cu / 8 * 8) : 8;
-    dim3 grid(args.tiles_total < resident ? args.tiles_total : resident), block(WM * WN * 64);
+    dim3 grid(total < resident ? total : resident), block(WM * WN * 64);
     hipLaunchKernelGGL(kern, grid, block, smem, st, args);
     g_gemm_bf16_launches++;
     return launch_status("gemm_bf16");
 }
 
 template <int EPI, bool OUT_F32>
-int launch_epi(int variant, ProbPair& args, int n, hipStream_t st) {
+int launch_epi(int variant, ProbSet& args, int n, hipStream_t st) {
     switch (variant) {
         case 4: return launch_cfg<256, 256, 2, 4, 2, EPI, OUT_F32>(args, n, st);
         case 1: return launch_cfg<128, 128, 2, 2, 4, EPI, OUT_F32>(args, n, st);
@@ -415,8 +417,8 @@ long long g_gemm_bf16_launches = 0;
 int g_gemm_bf16_variant = -1;  // -1: choose by shape; 0 / 4: forced 128x128 / 256x256 tiles (sd3_gemm_bf16_force_tile); 1: 128x128 with a ring of four stages
 
 int gemm_bf16_grouped(const GemmBf16Problem* probs, int n, int out_is_f32, int epi, hipStream_t st) {
-    if (n < 1 || n > 2) return fail(SD3_ERR_INVALID_ARG, "gemm_bf16_grouped: 1 or 2 problems (got %d)", n);
-    ProbPair args{};
+    if (n < 1 || n > MAX_PROBS) return fail(SD3_ERR_INVALID_ARG, "gemm_bf16_grouped: 1 to %d problems (got %d)", MAX_PROBS, n);
+    ProbSet args{};
     int m = 0, max_M = 0;
     for (int i = 0; i < n; i++) {
         const GemmBf16Problem& q = probs[i];
@@ -436,7 +438,7 @@ int gemm_bf16_grouped(const GemmBf16Problem* probs, int n, int out_is_f32, int e
         if (q.M > max_M) max_M = q.M;
     }
     if (m == 0) return SD3_OK;
-    auto launch = [&](ProbPair& pp, int count, int v) -> int {
+    auto launch = [&](ProbSet& pp, int count, int v) -> int {
 #define SD3_GEMM_BF16_LAUNCH(E) return out_is_f32 ? launch_epi<E, true>(v, pp, count, st) : launch_epi<E, false>(v, pp, count, st)
         switch (epi) {
             case EPI_BIAS: SD3_GEMM_BF16_LAUNCH(EPI_BIAS);
@@ -462,22 +464,28 @@ int gemm_bf16_grouped(const GemmBf16Problem* probs, int n, int out_is_f32, int e
         for (int i = 0; i < m; i++) tiles128 += ((args.p[i].M + 127) / 128) * ((args.p[i].N + 127) / 128);
         if (tiles128 <= cus) v = 1;
     }
-    if (m == 2 && v == 4) {
-        // A persistent launch takes ceil(tiles / compute units) rounds of tile time. When the small problem's tiles push the
-        // pair into one more round than the large problem needs alone, the small one goes first in a launch of its own with
-        // small tiles (a short single round) instead of costing a whole round of large tiles.
+    if (m >= 2 && v == 4) {
+        // A persistent launch takes ceil(tiles / compute units) rounds of tile time. When the tiles of the problems with few
+        // rows push the group into one more round than the large problems need alone, the small ones go first in a launch of
+        // their own with small tiles (a short single round) instead of costing a whole round of large tiles.
         const int cus = compute_units();
         if (cus <= 0) return SD3_ERR_HIP;
-        auto tiles256 = [](const Prob& q) { return ((q.M + 255) / 256) * ((q.N + 255) / 256); };
-        const int big = args.p[0].M >= args.p[1].M ? 0 : 1, small = 1 - big;
-        const int t_big = tiles256(args.p[big]), t_both = t_big + tiles256(args.p[small]);
-        if (args.p[small].M < 1024 && (t_both + cus - 1) / cus > (t_big + cus - 1) / cus) {
-            ProbPair one{};
-            one.p[0] = args.p[small];
-            const int small_tiles = ((one.p[0].M + 127) / 128) * ((one.p[0].N + 127) / 128);
-            SD3_TRY(launch(one, 1, small_tiles <= cus ? 1 : 0));
-            one.p[0] = args.p[big];
-            return launch(one, 1, 4);
+        auto tiles = [](const Prob& q, int t) { return ((q.M + t - 1) / t) * ((q.N + t - 1) / t); };
+        ProbSet big{}, small{};
+        int nb = 0, ns = 0, t_big = 0, t_small = 0, t_small128 = 0;
+        for (int i = 0; i < m; i++) {
+            if (args.p[i].M < 1024) {
+                small.p[ns++] = args.p[i];
+                t_small += tiles(args.p[i], 256);
+                t_small128 += tiles(args.p[i], 128);
+            } else {
+                big.p[nb++] = args.p[i];
+                t_big += tiles(args.p[i], 256);
+            }
+        }
+        if (ns > 0 && nb > 0 && (t_big + t_small + cus - 1) / cus > (t_big + cus - 1) / cus) {
+            SD3_TRY(launch(small, ns, t_small128 <= cus ? 1 : 0));
+            return launch(big, nb, 4);
         }
     }
     return launch(args, m, v);
