@@ -1,0 +1,98 @@
+"""Stand-in for the reference's torch extension `custom_modules` (PYBIND11_MODULE, modules.cpp:1789-1815), forward entry
+points only, so that scripts written like the reference's drivers run against this library unchanged:
+
+    import sys; sys.path.insert(0, "<repo>/sd3.c_amd"); import custom_modules as F
+    x_out = F.DiT(pooled, captions, latent, timesteps, params, num_layers, set(dual_layers), pooled_dim, captions_dim,
+                  in_channels, emb_dim, attn_heads, mlp_expand, patch_size, pos_embed_max_size, base_height, use_qk_norm)
+
+The reference's `Dit_block` and `DiT` take host tensors and compute on the CPU (module_tests/DiT.py:33-47,
+module_tests/dit_block.py:40-46); here the same calls copy their arguments to the GPU, run the fp32 path (the one held to
+the reference's 1e-4 / 1e-5 comparisons) and copy the results back, keeping the in-place contract of the block:
+`context_embeddings` and `latent_vector` are overwritten and returned. `DiT_block_cuda` takes device tensors as in
+module_tests/dit_block.py:60-66. There is no CPU fallback: without a GPU every call raises.
+
+The backward functions and `softmax*` of the extension are not on the forward path and are not provided.
+"""
+import os
+import sys
+
+import torch
+
+_here = os.path.dirname(os.path.abspath(__file__))
+if "sd3_c_amd" not in sys.modules:  # the package directory name has a dot in it: load it under an importable name
+    import importlib.util
+
+    _spec = importlib.util.spec_from_file_location("sd3_c_amd", os.path.join(_here, "__init__.py"), submodule_search_locations=[_here])
+    _mod = importlib.util.module_from_spec(_spec)
+    sys.modules["sd3_c_amd"] = _mod
+    _spec.loader.exec_module(_mod)
+from sd3_c_amd import modules as _M  # noqa: E402
+
+_DEV = "cuda"
+
+
+def _up(t):
+    return t.detach().to(device=_DEV, dtype=torch.float32).contiguous()
+
+
+def _params_up(params):
+    return {k: _up(v) for k, v in params.items()}
+
+
+def _host_op(fn):
+    """Operator-level entry points: host tensors in, host tensor out, like the reference's CPU functions."""
+    def wrapped(*args):
+        dev_args = [_up(a) if isinstance(a, torch.Tensor) else a for a in args]
+        out = fn(*dev_args)
+        torch.cuda.synchronize()
+        if isinstance(out, (list, tuple)):
+            return [o.cpu() if isinstance(o, torch.Tensor) else o for o in out]
+        return out.cpu() if isinstance(out, torch.Tensor) else out
+    wrapped.__name__ = fn.__name__
+    wrapped.__doc__ = fn.__doc__
+    return wrapped
+
+
+layer_norm = _host_op(lambda input, weight=None, bias=None, eps=1e-5, save_for_backward=False: _M.layer_norm(input, weight, bias, eps, save_for_backward))
+rms_norm = _host_op(lambda input, weight, eps, save_for_backward=False: _M.rms_norm(input, weight, eps, save_for_backward))
+gelu = _host_op(_M.gelu_tanh)
+silu = _host_op(_M.silu)
+linear = _host_op(_M.linear)
+conv2d = _host_op(_M.conv2d)
+sinusoidal_embedding = _host_op(_M.sinusoidal_embedding)
+mha = _host_op(_M.mha)
+mlp = _host_op(_M.mlp)
+
+
+def positional_embedding(emb_dim, height, width, base_size):
+    """modules.cpp:997 positional_embedding2D_forward"""
+    out = _M.positional_embedding(emb_dim, height, width, base_size, device=_DEV)
+    torch.cuda.synchronize()
+    return out.cpu()
+
+
+def Dit_block(temp_embeddings, context_embeddings, latent_vector, params, B, Tc, Tx, emb_dim, attn_heads, mlp_expand, use_dual_attention, use_qk_norm,
+              discard_context):
+    """modules.cpp:1508 DiT_block_forward on host tensors: context_embeddings and latent_vector are updated in place and returned."""
+    y, c, x = _up(temp_embeddings), _up(context_embeddings), _up(latent_vector)
+    c, x = _M.Dit_block(y, c, x, _params_up(params), B, Tc, Tx, emb_dim, attn_heads, mlp_expand, use_dual_attention, use_qk_norm, discard_context,
+                        precision="fp32")
+    context_embeddings.copy_(c.to(context_embeddings.device))
+    latent_vector.copy_(x.to(latent_vector.device))
+    return [context_embeddings, latent_vector]
+
+
+def DiT_block_cuda(temp_embeddings, context_embeddings, latent_vector, params, B, Tc, Tx, emb_dim, attn_heads, mlp_expand, use_dual_attention,
+                   use_qk_norm, discard_context):
+    """modules.cpp:1783 DiT_block_forward_cuda: device tensors, updated in place and returned."""
+    return _M.Dit_block(temp_embeddings, context_embeddings, latent_vector, params, B, Tc, Tx, emb_dim, attn_heads, mlp_expand, use_dual_attention,
+                        use_qk_norm, discard_context, precision="fp32")
+
+
+def DiT(pooled_captions, captions, latent_vector, timesteps, params, num_layers, dual_attention_layers, pooled_dim, captions_dim, C_in, emb_dim, attn_heads,
+        mlp_expand, patch_size, pos_embed_max_size, base_height, use_qk_norm):
+    """modules.cpp:1605 DiT_forward on host (or device) tensors: returns a new (B, C_in, H, W) tensor on the latent's device."""
+    out = _M.DiT(_up(pooled_captions), _up(captions), _up(latent_vector), _up(timesteps), _params_up(params), num_layers, dual_attention_layers,
+                 pooled_dim, captions_dim, C_in, emb_dim, attn_heads, mlp_expand, patch_size, pos_embed_max_size, base_height, use_qk_norm,
+                 precision="fp32")
+    return out.to(latent_vector.device)

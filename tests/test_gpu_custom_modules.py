@@ -1,0 +1,60 @@
+"""The stand-in for the reference's `custom_modules` extension (sd3.c_amd/custom_modules.py), used the way the reference's
+own drivers use the extension: host tensors, the reference's argument lists, in-place update of the block's streams."""
+import os
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import cases
+from gpu_util import max_abs, F32_TOL
+
+pytestmark = pytest.mark.gpu
+HERE = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(os.path.dirname(HERE), "sd3.c_amd"))
+import custom_modules as F  # noqa: E402
+
+GOLDEN = np.load(os.path.join(HERE, "golden", "reference_outputs.npz"))
+
+
+def test_dit_called_like_module_tests_DiT_py():
+    """module_tests/DiT.py:33-49 with the inputs of the committed golden vector: host tensors in, host tensor out."""
+    k = cases.dit_reference_test_case()
+    cfg = k["cfg"]
+    params = {n: torch.from_numpy(v) for n, v in k["params"].items()}
+    latent, captions = torch.from_numpy(k["latent"]), torch.from_numpy(k["captions"])
+    pooled, timesteps = torch.from_numpy(k["pooled"]), torch.from_numpy(k["timesteps"])
+    x_out = F.DiT(pooled, captions, latent, timesteps, params, cfg.num_layers, set(cfg.dual_attention_layers), cfg.pooled_dim, cfg.captions_dim,
+                  cfg.in_channels, cfg.emb_dim, cfg.attn_heads, cfg.mlp_expand, cfg.patch_size, cfg.pos_embed_max_size, cfg.base_height, cfg.use_qk_norm)
+    assert x_out.device.type == "cpu" and x_out.shape == latent.shape
+    gold = np.load(os.path.join(HERE, "golden", "reference_dit_test_config.npz"))["out"]
+    assert max_abs(x_out.numpy(), gold) <= F32_TOL
+
+
+@pytest.mark.parametrize("name", list(cases.BLOCK_CASES)[:2])
+def test_block_called_like_module_tests_dit_block_py(name):
+    """module_tests/dit_block.py:40-46 and :60-66: the host call and the device call update c and x in place."""
+    k = cases.block_case(name)
+    (B, Tc, C), Tx = k["c"].shape, k["x"].shape[1]
+    params = {n: torch.from_numpy(v) for n, v in k["params"].items()}
+    y, c, x = torch.from_numpy(k["y"].copy()), torch.from_numpy(k["c"].copy()), torch.from_numpy(k["x"].copy())
+    c_out, x_out = F.Dit_block(y, c, x, params, B, Tc, Tx, C, k["NH"], k["mlp_expand"], k["use_dual"], k["use_qk_norm"], k["discard_context"])
+    assert c_out is c and x_out is x
+    assert max_abs(x.numpy(), GOLDEN[name + ".x"]) <= F32_TOL
+    if not k["discard_context"]:
+        assert max_abs(c.numpy(), GOLDEN[name + ".c"]) <= F32_TOL
+    yd, cd, xd = (torch.from_numpy(k[n].copy()).cuda() for n in ("y", "c", "x"))
+    c2, x2 = F.DiT_block_cuda(yd, cd, xd, {n: v.cuda() for n, v in params.items()}, B, Tc, Tx, C, k["NH"], k["mlp_expand"], k["use_dual"], k["use_qk_norm"],
+                              k["discard_context"])
+    assert x2 is xd and torch.equal(xd.cpu(), x)
+
+
+def test_operator_entry_points_take_host_tensors():
+    x = torch.randn(2, 5, 64)
+    out = F.layer_norm(x, None, None, 1e-6, False)[0]
+    assert out.device.type == "cpu"
+    assert float((out - torch.nn.functional.layer_norm(x, (64,), eps=1e-6)).abs().max()) <= F32_TOL
+    assert float((F.gelu(x) - torch.nn.functional.gelu(x, approximate="tanh")).abs().max()) <= F32_TOL
+    W, b = torch.randn(64, 32) * 0.1, torch.randn(32)
+    assert float((F.linear(x, W, b) - (x @ W + b)).abs().max()) <= F32_TOL
