@@ -130,6 +130,16 @@ int sd3_dit_forward(sd3_ctx* ctx, const float* pooled, const float* captions, co
                     int emb_dim, int attn_heads, int mlp_expand, int patch_size, int pos_embed_max_size, int base_height, int use_qk_norm,
                     int precision);
 
+/* The sampler step around the denoiser, with no counterpart in the reference (which stops at the velocity): the same
+ * forward on a batch laid out [B/2 unconditional ; B/2 conditional] samples (both halves of `latent` hold the same B/2
+ * latents), with classifier-free guidance and one Euler step of the flow-matching sampler applied where the tokens go
+ * back to pixels:  latent_out[i] = latent[i] + dsigma * (v_u[i] + guidance * (v_c[i] - v_u[i])),  i < B/2,
+ * dsigma = sigma_next - sigma. latent_out is (B/2, C_in, H, W) and must not alias latent. */
+int sd3_dit_forward_cfg_euler(sd3_ctx* ctx, const float* pooled, const float* captions, const float* latent, const float* timesteps, float* latent_out,
+                              int B, int Tc, int H, int W, int num_layers, const int* dual_attention_layers, int n_dual, int pooled_dim, int captions_dim,
+                              int C_in, int emb_dim, int attn_heads, int mlp_expand, int patch_size, int pos_embed_max_size, int base_height,
+                              int use_qk_norm, int precision, float guidance, float dsigma);
+
 /* Per-kernel-class timing (no counterpart in the reference, which has no profiling). Between begin and end every
  * launch made through `ctx` by sd3_dit_block* / sd3_dit_forward is bracketed by two HIP events on the context's stream.
  * sd3_profile_end synchronises and returns, per class, the summed event time in ms, the summed algorithmic work

@@ -151,6 +151,8 @@ int conv2d_direct(const float* in, float* out, const float* kernel, const float*
 int im2col_patches(const float* latent, void* out, int out_bf16, int B, int Cin, int H, int W, int p, hipStream_t st);
 // tokens (B, h*w, p*p*Cin) -> pixels (B,Cin,H,W)
 int unpatchify(const float* tokens, float* out, int B, int Cin, int H, int W, int p, hipStream_t st);
+int unpatchify_cfg_euler(const float* tokens, const float* latent, float* out, int n_samples, int Cin, int H, int W, int p, float guidance, float dsigma,
+                         hipStream_t st);
 
 // Small-M linear (M <= 8): out(M, N) = act(x(M,K) @ W[:, n0:n0+N] + b[n0:n0+N]); W fp32 (K, ldw) or bf16 (K, ldw), both N-contiguous.
 struct SmallLinearJob {

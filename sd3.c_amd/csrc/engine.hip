@@ -733,9 +733,15 @@ int sd3_dit_block(sd3_ctx* ctx, const float* y, float* c, float* x, const char* 
 }
 
 // ------------------------------------------------------------------ full forward
-int sd3_dit_forward(sd3_ctx* ctx, const float* pooled, const float* captions, const float* latent, const float* timesteps, float* out, int B, int Tc,
-                    int H, int W, int num_layers, const int* dual_attention_layers, int n_dual, int pooled_dim, int captions_dim, int C_in, int emb_dim,
-                    int attn_heads, int mlp_expand, int patch_size, int pos_embed_max_size, int base_height, int use_qk_norm, int precision) {
+// guidance step: null for the plain forward (out = velocity of every batch element); otherwise the batch is
+// [B/2 unconditional ; B/2 conditional] and out (B/2 samples) = latent + dsigma * (v_u + guidance * (v_c - v_u))
+struct CfgEulerStep {
+    float guidance, dsigma;
+};
+static int dit_forward_impl(sd3_ctx* ctx, const float* pooled, const float* captions, const float* latent, const float* timesteps, float* out, int B, int Tc,
+                            int H, int W, int num_layers, const int* dual_attention_layers, int n_dual, int pooled_dim, int captions_dim, int C_in,
+                            int emb_dim, int attn_heads, int mlp_expand, int patch_size, int pos_embed_max_size, int base_height, int use_qk_norm,
+                            int precision, const CfgEulerStep* step) {
     NOTNULL(ctx); NOTNULL(pooled); NOTNULL(captions); NOTNULL(latent); NOTNULL(timesteps); NOTNULL(out);
     SD3_REQUIRE(num_layers > 0 && patch_size > 0 && H >= patch_size && W >= patch_size && C_in > 0 && pooled_dim > 0 && captions_dim > 0 && attn_heads > 0 &&
                     emb_dim > 0 && n_dual >= 0 && (n_dual == 0 || dual_attention_layers),
@@ -894,9 +900,27 @@ int sd3_dit_forward(sd3_ctx* ctx, const float* pooled, const float* captions, co
         SD3_TRY(ln_mod(ctx, x, x_hid, nullptr, ada_out + C, ada_out, nullptr, nullptr, 2 * C, 1e-5f, B, Tx, C, bf));
         GemmEpilogueArgs none;
         SD3_TRY(linear_layer(ctx, precision, x_hid, out_w, out_b, tokens, 1, PPC, B * Tx, PPC, C, EPI_BIAS, none));
-        SD3_TRY(unpatchify(tokens, out, B, C_in, H, W, p, st));
+        if (step) SD3_TRY(unpatchify_cfg_euler(tokens, latent, out, B / 2, C_in, H, W, p, step->guidance, step->dsigma, st));
+        else SD3_TRY(unpatchify(tokens, out, B, C_in, H, W, p, st));
     }
     return SD3_OK;
+}
+
+int sd3_dit_forward(sd3_ctx* ctx, const float* pooled, const float* captions, const float* latent, const float* timesteps, float* out, int B, int Tc,
+                    int H, int W, int num_layers, const int* dual_attention_layers, int n_dual, int pooled_dim, int captions_dim, int C_in, int emb_dim,
+                    int attn_heads, int mlp_expand, int patch_size, int pos_embed_max_size, int base_height, int use_qk_norm, int precision) {
+    return dit_forward_impl(ctx, pooled, captions, latent, timesteps, out, B, Tc, H, W, num_layers, dual_attention_layers, n_dual, pooled_dim, captions_dim,
+                            C_in, emb_dim, attn_heads, mlp_expand, patch_size, pos_embed_max_size, base_height, use_qk_norm, precision, nullptr);
+}
+
+int sd3_dit_forward_cfg_euler(sd3_ctx* ctx, const float* pooled, const float* captions, const float* latent, const float* timesteps, float* latent_out,
+                              int B, int Tc, int H, int W, int num_layers, const int* dual_attention_layers, int n_dual, int pooled_dim, int captions_dim,
+                              int C_in, int emb_dim, int attn_heads, int mlp_expand, int patch_size, int pos_embed_max_size, int base_height,
+                              int use_qk_norm, int precision, float guidance, float dsigma) {
+    SD3_REQUIRE(B >= 2 && B % 2 == 0, "DiT guidance step: the batch holds [unconditional ; conditional] halves, so B must be even (got %d)", B);
+    const CfgEulerStep step{guidance, dsigma};
+    return dit_forward_impl(ctx, pooled, captions, latent, timesteps, latent_out, B, Tc, H, W, num_layers, dual_attention_layers, n_dual, pooled_dim,
+                            captions_dim, C_in, emb_dim, attn_heads, mlp_expand, patch_size, pos_embed_max_size, base_height, use_qk_norm, precision, &step);
 }
 
 // ------------------------------------------------------------------ bf16 kernels on their own

@@ -472,23 +472,42 @@ int im2col_patches(const float* latent, void* out, int out_bf16, int B, int Cin,
 }
 
 // modules.cpp:1730-1752: out[b, ch, hp*p+ph, wp*p+pw] = tokens[b, hp*Wp+wp, (ph*p+pw)*Cin + ch]
-__global__ void __launch_bounds__(256) unpatchify_kernel(const float* __restrict__ tokens, float* __restrict__ out, int B, int Cin, int H, int W, int p,
-                                                         int Hp, int Wp, long long n) {
+// CFG: the batch holds [n unconditional ; n conditional] samples and the kernel writes, for each of the n samples, the
+// latent after classifier-free guidance and one Euler step of the flow-matching sampler:
+//   out = latent + dsigma * (v_u + guidance * (v_c - v_u))          (no counterpart in the reference, which stops at v)
+template <bool CFG>
+__global__ void __launch_bounds__(256) unpatchify_kernel(const float* __restrict__ tokens, const float* __restrict__ latent, float* __restrict__ out,
+                                                         int B, int Cin, int H, int W, int p, int Hp, int Wp, long long n, float guidance, float dsigma) {
     long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= n) return;
     const int w = (int)(idx % W), h = (int)((idx / W) % H);
     const int ch = (int)((idx / ((long long)W * H)) % Cin), b = (int)(idx / ((long long)W * H * Cin));
     const int hp = h / p, ph = h % p, wq = w / p, pw = w % p;
-    float v = 0.f;
-    if (hp < Hp && wq < Wp) v = tokens[((long long)b * Hp * Wp + (long long)hp * Wp + wq) * (p * p * Cin) + (ph * p + pw) * Cin + ch];
-    out[idx] = v;
+    const bool inside = hp < Hp && wq < Wp;
+    const long long tok = ((long long)hp * Wp + wq) * (p * p * Cin) + (ph * p + pw) * Cin + ch, per_sample = (long long)Hp * Wp * (p * p * Cin);
+    if (!CFG) {
+        out[idx] = inside ? tokens[(long long)b * per_sample + tok] : 0.f;
+    } else {
+        const float vu = inside ? tokens[(long long)b * per_sample + tok] : 0.f;
+        const float vc = inside ? tokens[(long long)(b + B) * per_sample + tok] : 0.f;
+        out[idx] = latent[idx] + dsigma * (vu + guidance * (vc - vu));
+    }
 }
 int unpatchify(const float* tokens, float* out, int B, int Cin, int H, int W, int p, hipStream_t st) {
     const int Hp = (H - p) / p + 1, Wp = (W - p) / p + 1;
     const long long n = (long long)B * Cin * H * W;
     if (n == 0) return SD3_OK;
-    hipLaunchKernelGGL(unpatchify_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, tokens, out, B, Cin, H, W, p, Hp, Wp, n);
+    hipLaunchKernelGGL(unpatchify_kernel<false>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, tokens, nullptr, out, B, Cin, H, W, p, Hp, Wp, n, 0.f, 0.f);
     return launch_status("unpatchify");
+}
+int unpatchify_cfg_euler(const float* tokens, const float* latent, float* out, int n_samples, int Cin, int H, int W, int p, float guidance, float dsigma,
+                         hipStream_t st) {
+    const int Hp = (H - p) / p + 1, Wp = (W - p) / p + 1;
+    const long long n = (long long)n_samples * Cin * H * W;
+    if (n == 0) return SD3_OK;
+    hipLaunchKernelGGL(unpatchify_kernel<true>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, tokens, latent, out, n_samples, Cin, H, W, p, Hp, Wp, n,
+                       guidance, dsigma);
+    return launch_status("unpatchify_cfg_euler");
 }
 
 }  // namespace sd3

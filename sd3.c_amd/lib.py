@@ -44,6 +44,7 @@ SIGNATURES = {
     "sd3_weights_prepare": [vp, ci],
     "sd3_dit_block": [vp, vp, vp, vp, cs] + [ci] * 10,
     "sd3_dit_forward": [vp] * 6 + [ci] * 5 + [vp] + [ci] * 12,
+    "sd3_dit_forward_cfg_euler": [vp] * 6 + [ci] * 5 + [vp] + [ci] * 12 + [cf, cf],
     "sd3_profile_begin": [vp],
     "sd3_profile_end": [vp, vp, vp, vp],
     "sd3_flash_attention_bf16": [vp] * 8 + [ci] * 5 + [vp],

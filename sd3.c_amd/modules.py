@@ -247,6 +247,25 @@ class Context:
                emb_dim, attn_heads, mlp_expand, patch_size, pos_embed_max_size, base_height, int(use_qk_norm), _PREC[precision])
         return out
 
+    def forward_cfg_euler(self, pooled_captions, captions, latent_vector, timesteps, guidance, dsigma, num_layers, dual_attention_layers, pooled_dim,
+                          captions_dim, C_in, emb_dim, attn_heads, mlp_expand, patch_size, pos_embed_max_size, base_height, use_qk_norm, precision="fp32",
+                          out=None):
+        """The forward on a batch [n unconditional ; n conditional] followed, in its last kernel, by classifier-free guidance and
+        one Euler step: returns latent[:n] + dsigma * (v_u + guidance * (v_c - v_u)), shape (n, C_in, H, W)."""
+        lat = _dev(latent_vector, "latent_vector")
+        B, _, H, W = lat.shape
+        Tc = captions.shape[1]
+        if out is None:
+            out = torch.empty((B // 2,) + tuple(lat.shape[1:]), device=lat.device)
+        dual = sorted(int(i) for i in dual_attention_layers)
+        arr = (C.c_int * max(1, len(dual)))(*dual)
+        L.call("sd3_ctx_set_stream", self._h, _stream())
+        L.call("sd3_dit_forward_cfg_euler", self._h, _p(_dev(pooled_captions, "pooled_captions")), _p(_dev(captions, "captions")), _p(lat),
+               _p(_dev(timesteps, "timesteps")), _p(_dev(out, "out")), B, Tc, H, W, num_layers, C.cast(arr, C.c_void_p), len(dual), pooled_dim, captions_dim,
+               C_in, emb_dim, attn_heads, mlp_expand, patch_size, pos_embed_max_size, base_height, int(use_qk_norm), _PREC[precision], float(guidance),
+               float(dsigma))
+        return out
+
     def synchronize(self):
         L.call("sd3_ctx_synchronize", self._h)
 
@@ -321,3 +340,10 @@ class Denoiser:
         return self.ctx.forward(pooled_captions, captions, latent_vector, timesteps, c.num_layers, c.dual_attention_layers, c.pooled_dim, c.captions_dim,
                                 c.in_channels, c.emb_dim, c.attn_heads, c.mlp_expand, c.patch_size, c.pos_embed_max_size, c.base_height, c.use_qk_norm,
                                 self.precision, out)
+
+    def cfg_euler_step(self, pooled_captions, captions, latent_pair, timesteps, guidance, dsigma, out=None):
+        """One sampler step: `latent_pair` is the current latents repeated for the [unconditional ; conditional] halves."""
+        c = self.cfg
+        return self.ctx.forward_cfg_euler(pooled_captions, captions, latent_pair, timesteps, guidance, dsigma, c.num_layers, c.dual_attention_layers,
+                                          c.pooled_dim, c.captions_dim, c.in_channels, c.emb_dim, c.attn_heads, c.mlp_expand, c.patch_size,
+                                          c.pos_embed_max_size, c.base_height, c.use_qk_norm, self.precision, out)

@@ -102,3 +102,28 @@ def test_dit_missing_parameter_is_reported():
     with pytest.raises(L_.Sd3Error) as e:
         run_gpu_dit(k, "fp32", P)
     assert e.value.status == 2 and "linear_out.weight" in str(e.value)
+
+
+def test_cfg_euler_step_equals_forward_then_formula():
+    """The guided Euler step writes latent + dsigma * (v_u + g * (v_c - v_u)) from the same velocities the plain forward
+    returns (closed form; the reference has no sampler), for an odd grid so that pixels outside the patch grid are covered."""
+    cfg = DiTConfig(num_layers=2, dual_attention_layers=(0,), pooled_dim=32, captions_dim=64, in_channels=16, emb_dim=128, attn_heads=2, mlp_expand=4,
+                    patch_size=2, pos_embed_max_size=16, base_height=16, use_qk_norm=True)
+    P = _synthetic_device_params(cfg, 21)
+    g = torch.Generator(device="cuda").manual_seed(22)
+    n, Tc, H, W = 2, 5, 11, 14
+    lat = torch.randn((n, cfg.in_channels, H, W), device="cuda", generator=g)
+    lat_pair = torch.cat([lat, lat], 0).contiguous()
+    captions = torch.randn((2 * n, Tc, cfg.captions_dim), device="cuda", generator=g)
+    pooled = torch.randn((2 * n, cfg.pooled_dim), device="cuda", generator=g)
+    t = torch.full((2 * n,), 700.0, device="cuda")
+    for precision in ("fp32", "bf16"):
+        den = M.Denoiser(P, cfg, precision)
+        v = den(pooled, captions, lat_pair, t)
+        got = den.cfg_euler_step(pooled, captions, lat_pair, t, guidance=4.5, dsigma=-0.03)
+        torch.cuda.synchronize()
+        want = lat + (-0.03) * (v[:n] + 4.5 * (v[n:] - v[:n]))
+        assert got.shape == lat.shape
+        assert float((got - want).abs().max()) <= 1e-5
+    with pytest.raises(Exception):
+        den.cfg_euler_step(pooled[:3], captions[:3], lat_pair[:3], t[:3], 4.5, -0.03)   # an odd batch has no two halves
