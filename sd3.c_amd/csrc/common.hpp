@@ -127,6 +127,19 @@ int patch_embed_direct(const float* latent, float* out, const float* kernel, con
 // LayerNorm without affine over the last axis + optional modulation: out = LN(x)*(1+scale[b])+shift[b]; a second modulated
 // output (shift2/scale2/out2) may be produced from the same normalised row. scale/shift rows have stride mod_ld.
 // out_bf16 selects bf16 (1) or fp32 (0) outputs.
+// LayerNorm (no affine) + optional modulation of one tensor (B, T, C) into one or two outputs; two such jobs with the same C
+// and eps (the two streams of a block) can share a launch
+struct LayerNormJob {
+    const float* x;
+    void* out;
+    void* out2;
+    const float* shift;
+    const float* scale;
+    const float* shift2;
+    const float* scale2;
+    int mod_ld, B, T;
+};
+int layernorm_modulate_pair(const LayerNormJob* jobs, int n, float eps, int C, int out_bf16, hipStream_t st);
 int layernorm_modulate(const float* x, void* out, void* out2, const float* shift, const float* scale, const float* shift2, const float* scale2,
                        int mod_ld, float eps, int B, int T, int C, int out_bf16, hipStream_t st);
 int layernorm_full(const float* x, float* y, float* mean, float* rstd, const float* w, const float* bias, float eps, long long rows, int C,

@@ -252,6 +252,18 @@ int ln_mod(sd3_ctx* ctx, const float* x, void* out, void* out2, const float* shi
     return layernorm_modulate(x, out, out2, shift, scale, shift2, scale2, mod_ld, eps, B, T, C, bf, ctx->stream);
 }
 
+// The LayerNorms of the latent and of the context stream at the same point of the block: one launch
+int ln_mod_pair(sd3_ctx* ctx, const LayerNormJob* jobs, int n, float eps, int C, int bf) {
+    double bytes = 0;
+    for (int i = 0; i < n; i++) {
+        const double e = (double)jobs[i].B * jobs[i].T * C;
+        bytes += e * 4 + e * (bf ? 2 : 4) * (jobs[i].out2 ? 2 : 1);
+    }
+    if (bytes == 0) return SD3_OK;
+    ProfScope ps(ctx, SD3_PROF_LAYERNORM, bytes);
+    return layernorm_modulate_pair(jobs, n, eps, C, bf, ctx->stream);
+}
+
 int attention(sd3_ctx* ctx, const AttnSegments& a, int B, int NH, int HS, bool bf) {
     const double Tq = a.Tq[0] + a.Tq[1], Tk = a.T[0] + a.T[1];
     ProfScope ps(ctx, SD3_PROF_ATTENTION, 4.0 * B * NH * Tq * Tk * HS);
@@ -310,9 +322,12 @@ int run_block(sd3_ctx* ctx, int prec, const float* y, float* c, float* x, const 
     //      the dual branch's input comes from the same normalised latent rows
     const float* c_shift = d.discard ? cchunk(1) : cchunk(0);
     const float* c_scale = d.discard ? cchunk(0) : cchunk(1);
-    if (mc > 0) SD3_TRY(ln_mod(ctx, c, c_hid, nullptr, c_shift, c_scale, nullptr, nullptr, ldc_ada, 1e-6f, B, Tc, C, bf));
-    SD3_TRY(ln_mod(ctx, x, x_hid, d.dual ? x_hid2 : nullptr, xchunk(0), xchunk(1), d.dual ? xchunk(6) : nullptr, d.dual ? xchunk(7) : nullptr, ldx_ada,
-                   1e-6f, B, Tx, C, bf));
+    {
+        const LayerNormJob ln1[2] = {{x, x_hid, d.dual ? x_hid2 : nullptr, xchunk(0), xchunk(1), d.dual ? xchunk(6) : nullptr, d.dual ? xchunk(7) : nullptr,
+                                      ldx_ada, B, Tx},
+                                     {c, c_hid, nullptr, c_shift, c_scale, nullptr, nullptr, ldc_ada, B, Tc}};
+        SD3_TRY(ln_mod_pair(ctx, ln1, 2, 1e-6f, C, bf));
+    }
     {
         // bf16 path: the per-head RMSNorm of q and k (modules.cpp:1396-1399, 1420-1423) runs in the projection's epilogue, on the
         // fp32 accumulators, so the attention kernel streams K tiles straight into LDS
@@ -372,8 +387,11 @@ int run_block(sd3_ctx* ctx, int prec, const float* y, float* c, float* x, const 
 
     // ---- MLPs of both streams (modules.cpp:1463-1476, 1488-1504)
     const int mcm = d.discard ? 0 : mc;
-    if (mcm > 0) SD3_TRY(ln_mod(ctx, c, c_hid, nullptr, cchunk(3), cchunk(4), nullptr, nullptr, ldc_ada, 1e-6f, B, Tc, C, bf));
-    SD3_TRY(ln_mod(ctx, x, x_hid, nullptr, xchunk(3), xchunk(4), nullptr, nullptr, ldx_ada, 1e-6f, B, Tx, C, bf));
+    {
+        const LayerNormJob ln2[2] = {{x, x_hid, nullptr, xchunk(3), xchunk(4), nullptr, nullptr, ldx_ada, B, Tx},
+                                     {c, c_hid, nullptr, cchunk(3), cchunk(4), nullptr, nullptr, ldc_ada, B, d.discard ? 0 : Tc}};
+        SD3_TRY(ln_mod_pair(ctx, ln2, 2, 1e-6f, C, bf));
+    }
     {
         LayerCall up[2] = {{x_hid, w.x_mlp_w1, w.x_mlp_b1, x_mlp, d.E * C, mx, d.E * C, C, none},
                            {c_hid, w.c_mlp_w1, w.c_mlp_b1, c_mlp, d.E * C, mcm, d.E * C, C, none}};

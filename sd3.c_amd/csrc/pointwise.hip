@@ -27,16 +27,35 @@ __device__ __forceinline__ void store1<bf16_t>(bf16_t* p, float a) { *p = f32_to
 
 // One wavefront per row, the row held in registers (NV float4 per lane), two-pass mean / variance like the
 // reference (modules.cpp:22-37), then up to two modulated outputs (modules.cpp:1207-1221 fused in).
+template <typename OutT>
+struct LnSegDev {
+    const float* x;
+    OutT* out;
+    OutT* out2;
+    const float* shift;
+    const float* scale;
+    const float* shift2;
+    const float* scale2;
+    int mod_ld, T;
+    long long rows;
+};
+template <typename OutT>
+struct LnSegPair {
+    LnSegDev<OutT> s[2];  // rows [0, s[0].rows) belong to the first tensor, the rest to the second (the two streams of a block)
+};
 template <typename OutT, int NV>
-__global__ void __launch_bounds__(256) ln_mod_vec_kernel(const float* __restrict__ x, OutT* __restrict__ out, OutT* __restrict__ out2,
-                                                         const float* __restrict__ shift, const float* __restrict__ scale,
-                                                         const float* __restrict__ shift2, const float* __restrict__ scale2, int mod_ld, float eps,
-                                                         long long rows, int T, int C) {
+__global__ void __launch_bounds__(256) ln_mod_vec_kernel(const LnSegPair<OutT> segs, float eps, int C) {
     const int lane = threadIdx.x & (WAVE - 1);
-    const long long row = (long long)blockIdx.x * (blockDim.x / WAVE) + (threadIdx.x / WAVE);
-    if (row >= rows) return;
+    long long row = (long long)blockIdx.x * (blockDim.x / WAVE) + (threadIdx.x / WAVE);
+    const int which = row >= segs.s[0].rows ? 1 : 0;
+    if (which) row -= segs.s[0].rows;
+    const LnSegDev<OutT>& g = segs.s[which];
+    if (row >= g.rows) return;
+    const int T = g.T, mod_ld = g.mod_ld;
+    OutT* __restrict__ out = g.out;
+    OutT* __restrict__ out2 = g.out2;
     const int nvec = C >> 2;
-    const float4* xr = reinterpret_cast<const float4*>(x + row * C);
+    const float4* xr = reinterpret_cast<const float4*>(g.x + row * C);
     float4 v[NV];
     float s = 0.f;
 #pragma unroll
@@ -57,10 +76,10 @@ __global__ void __launch_bounds__(256) ln_mod_vec_kernel(const float* __restrict
     }
     const float rstd = 1.0f / sqrtf(wave_sum(q) / C + eps);
     const long long b = row / T;
-    const float4* sh = shift ? reinterpret_cast<const float4*>(shift + b * mod_ld) : nullptr;
-    const float4* sc = scale ? reinterpret_cast<const float4*>(scale + b * mod_ld) : nullptr;
-    const float4* sh2 = shift2 ? reinterpret_cast<const float4*>(shift2 + b * mod_ld) : nullptr;
-    const float4* sc2 = scale2 ? reinterpret_cast<const float4*>(scale2 + b * mod_ld) : nullptr;
+    const float4* sh = g.shift ? reinterpret_cast<const float4*>(g.shift + b * mod_ld) : nullptr;
+    const float4* sc = g.scale ? reinterpret_cast<const float4*>(g.scale + b * mod_ld) : nullptr;
+    const float4* sh2 = g.shift2 ? reinterpret_cast<const float4*>(g.shift2 + b * mod_ld) : nullptr;
+    const float4* sc2 = g.scale2 ? reinterpret_cast<const float4*>(g.scale2 + b * mod_ld) : nullptr;
 #pragma unroll
     for (int i = 0; i < NV; i++) {
         int j = lane + i * WAVE;
@@ -118,38 +137,68 @@ __global__ void __launch_bounds__(256) ln_mod_generic_kernel(const float* __rest
 }
 
 template <typename OutT>
-static int ln_mod_dispatch(const float* x, OutT* out, OutT* out2, const float* shift, const float* scale, const float* shift2, const float* scale2,
-                           int mod_ld, float eps, long long rows, int T, int C, hipStream_t st) {
+static bool ln_seg_vectorisable(const LnSegDev<OutT>& g, int C) {
+    auto al = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+    return (C % 4 == 0) && (C <= 2048) && (g.mod_ld % 4 == 0) && al(g.x) && al(g.out) && al(g.out2) && al(g.shift) && al(g.scale) && al(g.shift2) &&
+           al(g.scale2);
+}
+template <typename OutT>
+static int ln_mod_launch_vec(const LnSegPair<OutT>& segs, float eps, int C, hipStream_t st) {
     const int wpb = 4;
+    const long long rows = segs.s[0].rows + segs.s[1].rows;
     dim3 grid((unsigned)((rows + wpb - 1) / wpb)), block(wpb * WAVE);
-    const bool vec = (C % 4 == 0) && (C <= 2048) && (mod_ld % 4 == 0) && ((reinterpret_cast<uintptr_t>(x) & 15) == 0) &&
-                     ((reinterpret_cast<uintptr_t>(out) & 15) == 0) && ((reinterpret_cast<uintptr_t>(out2) & 15) == 0) &&
-                     ((reinterpret_cast<uintptr_t>(shift) & 15) == 0) && ((reinterpret_cast<uintptr_t>(scale) & 15) == 0) &&
-                     ((reinterpret_cast<uintptr_t>(shift2) & 15) == 0) && ((reinterpret_cast<uintptr_t>(scale2) & 15) == 0);
-    if (vec) {
-        const int nv = (C / 4 + WAVE - 1) / WAVE;
-#define SD3_LN_CASE(N)                                                                                                                    \
-    case N:                                                                                                                               \
-        hipLaunchKernelGGL((ln_mod_vec_kernel<OutT, N>), grid, block, 0, st, x, out, out2, shift, scale, shift2, scale2, mod_ld, eps, rows, T, C); \
+    const int nv = (C / 4 + WAVE - 1) / WAVE;
+#define SD3_LN_CASE(N)                                                                       \
+    case N:                                                                                  \
+        hipLaunchKernelGGL((ln_mod_vec_kernel<OutT, N>), grid, block, 0, st, segs, eps, C); \
         break;
-        switch (nv) {
-            SD3_LN_CASE(1) SD3_LN_CASE(2) SD3_LN_CASE(3) SD3_LN_CASE(4) SD3_LN_CASE(5) SD3_LN_CASE(6) SD3_LN_CASE(7) SD3_LN_CASE(8)
-        }
+    switch (nv) { SD3_LN_CASE(1) SD3_LN_CASE(2) SD3_LN_CASE(3) SD3_LN_CASE(4) SD3_LN_CASE(5) SD3_LN_CASE(6) SD3_LN_CASE(7) SD3_LN_CASE(8) }
 #undef SD3_LN_CASE
-    } else {
-        hipLaunchKernelGGL((ln_mod_generic_kernel<OutT>), grid, block, 0, st, x, out, out2, shift, scale, shift2, scale2, mod_ld, nullptr, nullptr,
-                           nullptr, nullptr, eps, rows, T, C);
-    }
     return launch_status("layernorm_modulate");
+}
+template <typename OutT>
+static int ln_mod_dispatch(const LnSegDev<OutT>& g, float eps, int C, hipStream_t st) {
+    if (g.rows == 0) return SD3_OK;
+    if (ln_seg_vectorisable(g, C)) {
+        LnSegPair<OutT> segs{};
+        segs.s[0] = g;
+        return ln_mod_launch_vec(segs, eps, C, st);
+    }
+    const int wpb = 4;
+    dim3 grid((unsigned)((g.rows + wpb - 1) / wpb)), block(wpb * WAVE);
+    hipLaunchKernelGGL((ln_mod_generic_kernel<OutT>), grid, block, 0, st, g.x, g.out, g.out2, g.shift, g.scale, g.shift2, g.scale2, g.mod_ld, nullptr, nullptr,
+                       nullptr, nullptr, eps, g.rows, g.T, C);
+    return launch_status("layernorm_modulate");
+}
+template <typename OutT>
+static int ln_mod_pair_t(const LayerNormJob* jobs, int n, float eps, int C, hipStream_t st) {
+    LnSegDev<OutT> g[2];
+    int m = 0;
+    for (int i = 0; i < n; i++) {
+        const LayerNormJob& j = jobs[i];
+        const long long rows = (long long)j.B * j.T;
+        if (rows == 0) continue;
+        g[m++] = LnSegDev<OutT>{j.x, (OutT*)j.out, (OutT*)j.out2, j.shift, j.scale, j.shift2, j.scale2, j.mod_ld, j.T, rows};
+    }
+    if (m == 2 && ln_seg_vectorisable(g[0], C) && ln_seg_vectorisable(g[1], C)) {
+        LnSegPair<OutT> segs{};
+        segs.s[0] = g[0];
+        segs.s[1] = g[1];
+        return ln_mod_launch_vec(segs, eps, C, st);  // the few rows of the second tensor ride along instead of paying a launch
+    }
+    for (int i = 0; i < m; i++) SD3_TRY(ln_mod_dispatch(g[i], eps, C, st));
+    return SD3_OK;
 }
 
 int layernorm_modulate(const float* x, void* out, void* out2, const float* shift, const float* scale, const float* shift2, const float* scale2,
                        int mod_ld, float eps, int B, int T, int C, int out_bf16, hipStream_t st) {
-    const long long rows = (long long)B * T;
-    if (rows == 0) return SD3_OK;
-    if (out_bf16)
-        return ln_mod_dispatch<bf16_t>(x, (bf16_t*)out, (bf16_t*)out2, shift, scale, shift2, scale2, mod_ld, eps, rows, T, C, st);
-    return ln_mod_dispatch<float>(x, (float*)out, (float*)out2, shift, scale, shift2, scale2, mod_ld, eps, rows, T, C, st);
+    const LayerNormJob j{x, out, out2, shift, scale, shift2, scale2, mod_ld, B, T};
+    return layernorm_modulate_pair(&j, 1, eps, C, out_bf16, st);
+}
+
+int layernorm_modulate_pair(const LayerNormJob* jobs, int n, float eps, int C, int out_bf16, hipStream_t st) {
+    if (n < 1 || n > 2) return fail(SD3_ERR_INVALID_ARG, "layernorm_modulate_pair: 1 or 2 tensors (got %d)", n);
+    return out_bf16 ? ln_mod_pair_t<bf16_t>(jobs, n, eps, C, st) : ln_mod_pair_t<float>(jobs, n, eps, C, st);
 }
 
 int layernorm_full(const float* x, float* y, float* mean, float* rstd, const float* w, const float* bias, float eps, long long rows, int C,
