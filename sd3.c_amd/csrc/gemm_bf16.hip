@@ -452,43 +452,46 @@ int gemm_bf16_grouped(const GemmBf16Problem* probs, int n, int out_is_f32, int e
 #undef SD3_GEMM_BF16_LAUNCH
     };
     if (g_gemm_bf16_variant >= 0) return launch(args, m, g_gemm_bf16_variant);
-    // tile shape: 256x256 (8 wavefronts, one workgroup per compute unit) for large problems, 128x128 (4 wavefronts, two
-    // workgroups per compute unit) when there are few rows
-    int v = max_M >= 1024 ? 4 : 0;
-    if (v == 0) {
-        // few rows and no more 128x128 tiles than compute units: one workgroup per unit, so LDS can hold a ring of four
-        // stages, which is what counts when the launch is a single short round bound by load latency
-        const int cus = compute_units();
-        if (cus <= 0) return SD3_ERR_HIP;
-        int tiles128 = 0;
-        for (int i = 0; i < m; i++) tiles128 += ((args.p[i].M + 127) / 128) * ((args.p[i].N + 127) / 128);
-        if (tiles128 <= cus) v = 1;
-    }
-    if (m >= 2 && v == 4) {
-        // A persistent launch takes ceil(tiles / compute units) rounds of tile time. When the tiles of the problems with few
-        // rows push the group into one more round than the large problems need alone, the small ones go first in a launch of
-        // their own with small tiles (a short single round) instead of costing a whole round of large tiles.
-        const int cus = compute_units();
-        if (cus <= 0) return SD3_ERR_HIP;
-        auto tiles = [](const Prob& q, int t) { return ((q.M + t - 1) / t) * ((q.N + t - 1) / t); };
-        ProbSet big{}, small{};
-        int nb = 0, ns = 0, t_big = 0, t_small = 0, t_small128 = 0;
-        for (int i = 0; i < m; i++) {
-            if (args.p[i].M < 1024) {
-                small.p[ns++] = args.p[i];
-                t_small += tiles(args.p[i], 256);
-                t_small128 += tiles(args.p[i], 128);
-            } else {
-                big.p[nb++] = args.p[i];
-                t_big += tiles(args.p[i], 256);
-            }
-        }
-        if (ns > 0 && nb > 0 && (t_big + t_small + cus - 1) / cus > (t_big + cus - 1) / cus) {
-            SD3_TRY(launch(small, ns, t_small128 <= cus ? 1 : 0));
-            return launch(big, nb, 4);
+    // Tile shape and grouping by a small cost model. A persistent launch takes ceil(tiles / resident workgroups) rounds; the unit
+    // of cost is one round of 256x256 tiles (8 wavefronts, one workgroup per compute unit). Measured on full rounds, a round of
+    // 128x128 tiles (4 wavefronts, two workgroups per unit) takes 0.58 of that for a quarter of the outputs per tile, and a launch
+    // of its own for problems with few rows (a short round of small tiles, bound by per-tile overhead) about 0.38.
+    const int cus = compute_units();
+    if (cus <= 0) return SD3_ERR_HIP;
+    constexpr double ROUND128 = 0.58, SMALL_LAUNCH = 0.38;
+    auto tiles = [](const Prob& q, int t) { return ((q.M + t - 1) / t) * ((q.N + t - 1) / t); };
+    auto rounds = [](long long t, int slots) { return (double)((t + slots - 1) / slots); };
+    ProbSet big{}, small{};
+    int nb = 0, ns = 0;
+    long long big256 = 0, big128 = 0, small256 = 0, small128 = 0;
+    for (int i = 0; i < m; i++) {
+        if (args.p[i].M < 1024) {
+            small.p[ns++] = args.p[i];
+            small256 += tiles(args.p[i], 256);
+            small128 += tiles(args.p[i], 128);
+        } else {
+            big.p[nb++] = args.p[i];
+            big256 += tiles(args.p[i], 256);
+            big128 += tiles(args.p[i], 128);
         }
     }
-    return launch(args, m, v);
+    // only problems with few rows: small tiles; with no more tiles than compute units one workgroup per unit, so that LDS can hold
+    // a ring of four stages
+    const int v_small = small128 <= cus ? 1 : 0;
+    if (nb == 0) return launch(args, m, v_small);
+    const double together256 = rounds(big256 + small256, cus), together128 = ROUND128 * rounds(big128 + small128, 2 * cus);
+    double best = together256 <= together128 ? together256 : together128;
+    int plan = together256 <= together128 ? 0 : 1;  // 0/1: one launch with 256/128 tiles; 2/3: the small problems first, alone
+    if (ns > 0) {
+        const double apart256 = rounds(big256, cus) + SMALL_LAUNCH, apart128 = ROUND128 * rounds(big128, 2 * cus) + SMALL_LAUNCH;
+        if (apart256 < best) { best = apart256; plan = 2; }
+        if (apart128 < best) { best = apart128; plan = 3; }
+    }
+    if (plan >= 2) {
+        SD3_TRY(launch(small, ns, v_small));
+        return launch(big, nb, plan == 2 ? 4 : 0);
+    }
+    return launch(args, m, plan == 0 ? 4 : 0);
 }
 
 int gemm_bf16(const bf16_t* A, const bf16_t* Wp, void* out, int out_is_f32, int ldc, int M, int N, int K, int epi, const GemmEpilogueArgs& ea,
