@@ -7,7 +7,7 @@ from conftest import load_package
 pkg = load_package()
 from sd3_c_amd import modules as M  # noqa: E402
 
-F32_TOL = 1e-4  # max abs error of the fp32 GPU path against the CPU reference arithmetic (the bar of BASELINE.json)
+F32_TOL = 1e-4  # max abs error of the fp32 GPU path against the CPU reference arithmetic (the fp32 parity bar of this build)
 BF16_REL_L2 = 1e-2  # relative L2 of the bf16 path against the fp32 path
 
 

@@ -37,7 +37,7 @@ def _naive_joint_attention(qkv0, qkv1, rq, rk, B, T0, T1, NH, HS):
 @pytest.mark.parametrize("B,T0,T1,NH", [(2, 154, 4096, 24), (1, 154, 1024, 24), (2, 7, 130, 4), (1, 0 + 64, 0, 2), (1, 1, 63, 3),
                                         (1, 64, 64, 1), (1, 3, 62, 1), (1, 1, 0, 1), (2, 33, 224, 2), (1, 100, 29, 2), (1, 60, 133, 1)])
 def test_flash_attention_bf16(B, T0, T1, NH):
-    """BASELINE config 2 is the first case: B=2, 24 heads of 64, 154 text + 4096 image tokens, q/k/v ~ N(0,1). The small cases sit
+    """The headline attention shape is the first case: B=2, 24 heads of 64, 154 text + 4096 image tokens, q/k/v ~ N(0,1). The small cases sit
     on the edges of the 64-key tiles and 32-key halves (one tile exactly, one key into the next tile, a single key, a segment
     boundary inside a tile) and of the three-stage tile ring (1, 2, 3 and 4 tiles)."""
     HS, C = 64, NH * 64

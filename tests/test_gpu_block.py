@@ -1,5 +1,5 @@
 """One MMDiT-X block on the MI355X against the reference arithmetic: golden vectors of the compiled reference, the CPU
-oracle on the same seeded inputs, a float64 statement of the block at the size of BASELINE config 1, and the bf16 path
+oracle on the same seeded inputs, a float64 statement of the block at the reference-runnable size (B=1, 256 image + 77 text tokens, width 1536), and the bf16 path
 against the fp32 path."""
 import os
 
@@ -68,7 +68,7 @@ def test_block_fp32_width_1536_vs_oracle(dual, discard):
 
 @pytest.mark.parametrize("dual", [True, False])
 def test_block_fp32_baseline_config1_vs_float64(dual):
-    """BASELINE config 1 at full size (B=1, 256 image + 77 text tokens, width 1536): the CPU oracle needs a minute for this,
+    """The CPU-runnable benchmark configuration at full size (B=1, 256 image + 77 text tokens, width 1536): the CPU oracle needs a minute for this,
     so the check is against the float64 numpy statement of the block that tests/test_oracle.py pins to the oracle."""
     k = _wide_case(1, 77, 256, dual, False, 21)
     c, x = run_gpu_block(k)

@@ -1,5 +1,5 @@
 """Full denoiser forward on the MI355X: fp32 path against golden vectors of the compiled reference and the CPU oracle,
-bf16 path against the fp32 path at the SD3.5-medium shape (BASELINE config 3), and size-independent properties."""
+bf16 path against the fp32 path at the SD3.5-medium shape with a 512x512 image, and size-independent properties."""
 import os
 
 import numpy as np
@@ -67,7 +67,7 @@ def _inputs(cfg, B, Tc, H, W, seed):
 
 
 def test_dit_bf16_vs_fp32_sd35_medium_512px():
-    """BASELINE config 3: full SD3.5-medium shape (24 blocks, width 1536, 13 dual blocks), 64x64 latent = 1024 image tokens,
+    """Full SD3.5-medium shape (24 blocks, width 1536, 13 dual blocks), 64x64 latent = 1024 image tokens,
     154 text tokens, batch 2. The bf16 path must stay within relative L2 1e-2 of the fp32 path on the final velocity."""
     cfg = sd35_medium()
     P = _synthetic_device_params(cfg, 5)
