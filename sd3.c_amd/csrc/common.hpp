@@ -2,6 +2,8 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
+#include <atomic>
+
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
@@ -114,7 +116,7 @@ struct GemmBf16Problem {
     int ldc, M, N, K;
     GemmEpilogueArgs ea;
 };
-extern long long g_gemm_bf16_launches;  // kernels launched by the bf16 GEMM so far (for per-launch profile figures)
+extern std::atomic<long long> g_gemm_bf16_launches;  // kernels launched by the bf16 GEMM so far (for per-launch profile figures)
 int gemm_bf16_grouped(const GemmBf16Problem* probs, int n, int out_is_f32, int epi, hipStream_t st);
 // (K,N) fp32 row-major -> (N,K) bf16 row-major
 int pack_weight_bf16(const float* W, bf16_t* out, int K, int N, hipStream_t st);

@@ -133,7 +133,7 @@ struct ProfScope {
     int cls;
     double work;
     long long gemm_launches_before;  // one bracketed call may launch more than one GEMM kernel; the class counts kernels
-    ProfScope(sd3_ctx* c, int cls_, double work_) : ctx(c), cls(cls_), work(work_), gemm_launches_before(g_gemm_bf16_launches) {
+    ProfScope(sd3_ctx* c, int cls_, double work_) : ctx(c), cls(cls_), work(work_), gemm_launches_before(g_gemm_bf16_launches.load(std::memory_order_relaxed)) {
         if (!ctx->prof_on) return;
         auto get = [&]() -> hipEvent_t {
             hipEvent_t e = nullptr;
@@ -153,7 +153,7 @@ struct ProfScope {
     ~ProfScope() {
         if (!a || !b) return;
         (void)hipEventRecord(b, ctx->stream);
-        const long long kernels = g_gemm_bf16_launches - gemm_launches_before;
+        const long long kernels = g_gemm_bf16_launches.load(std::memory_order_relaxed) - gemm_launches_before;
         ctx->prof.push_back({a, b, cls, work, kernels > 1 ? kernels : 1});
     }
 };

@@ -398,7 +398,7 @@ int launch_cfg(ProbSet& args, int n, hipStream_t st) {
     const int resident = (cus * per_cu / 8 * 8) > 8 ? (cus * per_cu / 8 * 8) : 8;
     dim3 grid(total < resident ? total : resident), block(WM * WN * 64);
     hipLaunchKernelGGL(kern, grid, block, smem, st, args);
-    g_gemm_bf16_launches++;
+    g_gemm_bf16_launches.fetch_add(1, std::memory_order_relaxed);
     return launch_status("gemm_bf16");
 }
 
@@ -413,7 +413,7 @@ int launch_epi(int variant, ProbSet& args, int n, hipStream_t st) {
 
 }  // namespace
 
-long long g_gemm_bf16_launches = 0;
+std::atomic<long long> g_gemm_bf16_launches{0};
 int g_gemm_bf16_variant = -1;  // -1: choose by shape; 0 / 4: forced 128x128 / 256x256 tiles (sd3_gemm_bf16_force_tile); 1: 128x128 with a ring of four stages
 
 int gemm_bf16_grouped(const GemmBf16Problem* probs, int n, int out_is_f32, int epi, hipStream_t st) {
