@@ -270,12 +270,12 @@ __global__ void __launch_bounds__(NW * 64, 2) flash_attn_bf16_kernel(SegDev s, f
 #pragma unroll
         for (int j = 0; j < 2; j++) pf[qb][j].u = make_uint4(0u, 0u, 0u, 0u);
 
-    auto aux_frag = [&](int key_base) -> Frag {  // AUX rows for keys key_base + l32
-        Frag f;
-        f.u = make_uint4((key_base + l32 >= T) ? 0x3f803f80u : 0x00003f80u, 0u, 0u, 0u);
-        return f;
-    };
-    auto scores = [&](int qb, const Frag& aux) {
+    // AUX rows for keys key_base + l32: one persistent operand whose first register alone changes from unit to unit
+    Frag aux;
+    aux.u = make_uint4(0u, 0u, 0u, 0u);
+    const int first_masked = T - l32;  // key_base >= first_masked  <=>  key key_base + l32 lies beyond the sequence
+    auto scores = [&](int qb, int key_base) {
+        aux.u.x = (key_base >= first_masked) ? 0x3f803f80u : 0x00003f80u;
         sacc[qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(aux.v, negm_f[qb].v, zero, 0, 0, 0);
 #pragma unroll
         for (int ks = 0; ks < 4; ks++) sacc[qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[ks], qf[qb][ks].v, sacc[qb], 0, 0, 0);
@@ -374,7 +374,7 @@ __global__ void __launch_bounds__(NW * 64, 2) flash_attn_bf16_kernel(SegDev s, f
     }
     __syncthreads();
     load_k(0, 0);
-    scores(0, aux_frag(0));
+    scores(0, 0);
     int st_cur = 0, st_nxt = STAGE_BYTES, st_ld = 2 * STAGE_BYTES;  // stages of tiles t, t+1, t+2
 
     for (int t = 0; t < nt; t++) {
@@ -383,7 +383,7 @@ __global__ void __launch_bounds__(NW * 64, 2) flash_attn_bf16_kernel(SegDev s, f
         //      frees; scores of (t,0,1); then fetch K of half 1 ----
         pv(1, 0);
         load_v(st_cur, 0, 0);
-        scores(1, aux_frag(t * BKV));
+        scores(1, t * BKV);
         load_k(st_cur, 1);
         inc = probs(0);
         pv(1, 1);
@@ -393,7 +393,7 @@ __global__ void __launch_bounds__(NW * 64, 2) flash_attn_bf16_kernel(SegDev s, f
         // ---- step (t, 0, 1): PV of (t,0,0); scores of (t,1,0) ----
         lds_wait_first4(vfr);
         pv(0, 0);
-        scores(0, aux_frag(t * BKV + 32));
+        scores(0, t * BKV + 32);
         inc = probs(1);
         lds_wait_last4(vfr);
         pv(0, 1);
@@ -409,7 +409,7 @@ __global__ void __launch_bounds__(NW * 64, 2) flash_attn_bf16_kernel(SegDev s, f
         fetch_tile(st_ld);
         pv(1, 0);
         load_v(st_cur, 1, 0);
-        scores(1, aux_frag(t * BKV + 32));
+        scores(1, t * BKV + 32);
         load_k(st_nxt, 0);
         inc = probs(0);
         pv(1, 1);
@@ -419,7 +419,7 @@ __global__ void __launch_bounds__(NW * 64, 2) flash_attn_bf16_kernel(SegDev s, f
         // ---- step (t, 1, 1): PV of (t,1,0); scores of (t+1,0,0) ----
         lds_wait_first4(vfr);
         pv(0, 0);
-        scores(0, aux_frag(t * BKV + BKV));
+        scores(0, t * BKV + BKV);
         inc = probs(1);
         lds_wait_last4(vfr);
         pv(0, 1);
