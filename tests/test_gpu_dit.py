@@ -127,3 +127,42 @@ def test_cfg_euler_step_equals_forward_then_formula():
         assert float((got - want).abs().max()) <= 1e-5
     with pytest.raises(Exception):
         den.cfg_euler_step(pooled[:3], captions[:3], lat_pair[:3], t[:3], 4.5, -0.03)   # an odd batch has no two halves
+
+
+def test_warm_forward_is_graph_capturable_and_replays_bit_identically():
+    """After one warm-up call a forward makes no allocation, memset or host synchronisation, so it can be captured into a
+    HIP graph. The graph is replayed several times, with eager work and synchronisations in between, and every replay must
+    reproduce the eager result bit for bit (both precisions, the sampler-step variant included)."""
+    cfg = DiTConfig(num_layers=3, dual_attention_layers=(0, 1), pooled_dim=64, captions_dim=64, in_channels=16, emb_dim=128, attn_heads=2, mlp_expand=4,
+                    patch_size=2, pos_embed_max_size=32, base_height=16, use_qk_norm=True)
+    P = _synthetic_device_params(cfg, 31)
+    g = torch.Generator(device="cuda").manual_seed(32)
+    B, Tc, H, W = 2, 9, 24, 20
+    lat = torch.randn((B, cfg.in_channels, H, W), device="cuda", generator=g)
+    captions = torch.randn((B, Tc, cfg.captions_dim), device="cuda", generator=g)
+    pooled = torch.randn((B, cfg.pooled_dim), device="cuda", generator=g)
+    t = torch.full((B,), 300.0, device="cuda")
+    for precision in ("bf16", "fp32"):
+        den = M.Denoiser(P, cfg, precision)
+        out, step_out = torch.empty_like(lat), torch.empty_like(lat[:1])
+        for _ in range(2):
+            den(pooled, captions, lat, t, out=out)
+            den.cfg_euler_step(pooled, captions, lat, t, 3.0, -0.05, out=step_out)
+        torch.cuda.synchronize()
+        want, want_step = out.clone(), step_out.clone()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            den(pooled, captions, lat, t, out=out)
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            den(pooled, captions, lat, t, out=out)
+            den.cfg_euler_step(pooled, captions, lat, t, 3.0, -0.05, out=step_out)
+        for i in range(3):
+            out.zero_()
+            step_out.zero_()
+            (lat * 2).sum().item()        # eager work and a synchronisation between replays
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out, want) and torch.equal(step_out, want_step), (precision, i)
