@@ -66,12 +66,14 @@ def _inputs(cfg, B, Tc, H, W, seed):
                 timesteps=(rng.random((B,), dtype=np.float32) * 1000).astype(np.float32))
 
 
-def test_dit_bf16_vs_fp32_sd35_medium_512px():
-    """Full SD3.5-medium shape (24 blocks, width 1536, 13 dual blocks), 64x64 latent = 1024 image tokens,
-    154 text tokens, batch 2. The bf16 path must stay within relative L2 1e-2 of the fp32 path on the final velocity."""
+@pytest.mark.parametrize("side", [64, 128])
+def test_dit_bf16_vs_fp32_sd35_medium(side):
+    """Full SD3.5-medium shape (24 blocks, width 1536, 13 dual blocks), batch 2, 154 text tokens, with a 64x64 latent (512x512
+    image, 1024 image tokens) and with the benchmark's 128x128 latent (1024x1024 image, 4096 image tokens). The bf16 path must
+    stay within relative L2 1e-2 of the fp32 path on the final velocity."""
     cfg = sd35_medium()
     P = _synthetic_device_params(cfg, 5)
-    k = _inputs(cfg, 2, 154, 64, 64, 6)
+    k = _inputs(cfg, 2, 154, side, side, 6)
     o32 = run_gpu_dit(k, "fp32", P)
     o16 = run_gpu_dit(k, "bf16", P)
     assert np.isfinite(o32).all() and np.isfinite(o16).all()
