@@ -156,7 +156,6 @@ __global__ void __launch_bounds__(NW * 64, 2) flash_attn_bf16_kernel(SegDev s, f
     // a score block starts from AUX . NEGM, where AUX[key][k=0] = 1, AUX[key][k=1] = (key beyond the sequence),
     // NEGM[k=0][query] = -m_run (kept representable in bf16), NEGM[k=1][query] = -1e30 and everything else is zero.
     float m_run[2] = {0.f, 0.f}, l_run[2] = {0.f, 0.f};
-    const bf16x2_t ONES = {(__bf16)1.0f, (__bf16)1.0f};
     const uint32_t NEG_BIG_HI = pack_bf16x2(0.f, -1e30f);  // bf16(-1e30) in the upper half
     Frag negm_f[2];
 #pragma unroll
@@ -284,7 +283,9 @@ __global__ void __launch_bounds__(NW * 64, 2) flash_attn_bf16_kernel(SegDev s, f
 #pragma unroll
         for (int ks = 0; ks < 4; ks++) kf[ks] = *reinterpret_cast<const bf16x8_t*>(smem + stage_byte + koff[ks] + kb * 32 * 128);
     };
-    // probabilities of one unit -> bf16 P^T operands + this lane's sum of the rounded values
+    // probabilities of one unit -> bf16 P^T operands + this lane's sum of them (of the unrounded values, with plain
+    // additions: the bf16 dot-product instructions, one per packed pair, measure about 8 cycles each during which the
+    // matrix unit accepts nothing, while additions issue beside it for free)
     auto pack_probs = [&](const f32x16_t& pr, Frag (&out)[2]) -> float {
         float ls0 = 0.f, ls1 = 0.f;
 #pragma unroll
@@ -293,8 +294,8 @@ __global__ void __launch_bounds__(NW * 64, 2) flash_attn_bf16_kernel(SegDev s, f
 #pragma unroll
             for (int e = 0; e < 4; e++) {
                 w[e] = pack_bf16x2(pr[8 * j + 2 * e], pr[8 * j + 2 * e + 1]);
-                if (e & 1) ls1 = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, w[e]), ONES, ls1, false);
-                else ls0 = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, w[e]), ONES, ls0, false);
+                if (e & 1) ls1 += pr[8 * j + 2 * e] + pr[8 * j + 2 * e + 1];
+                else ls0 += pr[8 * j + 2 * e] + pr[8 * j + 2 * e + 1];
             }
             out[j].u = make_uint4(w[0], w[1], w[2], w[3]);
         }
