@@ -79,6 +79,22 @@ def cpu_baseline(cfg, flops_per_step):
                       f"= {rate / 1e9:.3f} GFLOP/s on 1 thread of {os.cpu_count()} visible cores; scaled by FLOP to the {flops_per_step / 1e12:.2f} TFLOP step"}
 
 
+def mfma_probe():
+    """What this device's matrix cores sustain on the instruction the GEMM and attention kernels use, issued back to back from
+    registers by every wavefront (no memory traffic): with zero operands, and with random ones. The device holds its power
+    limit by lowering the clock, so the second figure, not the published peak, is what a kernel working on real data can
+    approach; `roofline.frac` stays relative to the published peak."""
+    import ctypes
+    from sd3_c_amd import lib as L
+    out = {}
+    for key, rnd in (("zero_operands", 0), ("random_operands", 1)):
+        v = ctypes.c_double(0.0)
+        L.call("sd3_probe_mfma_bf16", rnd, 40000, ctypes.byref(v))
+        out[key] = round(v.value, 1)
+    out["unit"] = "TFLOP/s"
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -178,6 +194,8 @@ def main():
         "ms_per_step_profiled": round(dt_prof / a.steps * 1e3, 3) if dt_prof else None,
         "roofline": roofline, "kernels": kernels,
     }
+    if a.precision == "bf16":
+        res["mfma_probe"] = mfma_probe()
     if not a.no_cpu_baseline:
         res["cpu_baseline"] = cpu_baseline(cfg, total_f)
     print(json.dumps(res))

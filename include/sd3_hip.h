@@ -169,6 +169,13 @@ int sd3_cast_f32_to_bf16(const float* in, void* out, long long n, void* stream);
  * process. tile = 0: chosen per call from the problem sizes (the default); 128: 128x128 tiles, two workgroups per compute
  * unit; 256: 256x256 tiles, one workgroup per compute unit. Results do not depend on the choice. */
 int sd3_gemm_bf16_force_tile(int tile);
+/* Measurement aid with no counterpart in the reference: the rate (in TFLOP/s) at which the device's matrix cores run the
+ * bf16 instruction the GEMM and attention kernels are built on when every wavefront issues it back to back on operands held
+ * in registers (no memory or LDS traffic), with all-zero operands (random_operands = 0) or random ones (1). The two differ
+ * widely because the device keeps its power limit by lowering the clock; the second figure is the ceiling for a kernel that
+ * works on real data. Runs on the current device's default stream, allocates a small buffer for the duration of the call,
+ * and returns after `iters` iterations of 8 instructions per wavefront (40000 take about 15 ms). */
+int sd3_probe_mfma_bf16(int random_operands, int iters, double* tflops);
 
 #ifdef __cplusplus
 }

@@ -52,6 +52,7 @@ SIGNATURES = {
     "sd3_gemm_bf16": [vp, vp, vp, vp, ci, ci, ci, ci, vp],
     "sd3_cast_f32_to_bf16": [vp, vp, cll, vp],
     "sd3_gemm_bf16_force_tile": [ci],
+    "sd3_probe_mfma_bf16": [ci, ci, vp],
 }
 
 

@@ -137,3 +137,18 @@ def test_cast_rounds_to_nearest_even():
     out = torch.empty(100000, device="cuda", dtype=torch.bfloat16)
     L.call("sd3_cast_f32_to_bf16", x.data_ptr(), out.data_ptr(), x.numel(), None)
     assert torch.equal(out, x.bfloat16())
+
+
+def test_mfma_probe_reports_a_plausible_rate_and_rejects_bad_arguments():
+    """The register-only matrix-instruction loop must land between a tenth of the published bf16 peak and a little above
+    it (2.5 PFLOP/s at the maximum clock) for zero operands, and random operands must not be faster than zeros."""
+    import ctypes
+    z, r = ctypes.c_double(0.0), ctypes.c_double(0.0)
+    L.call("sd3_probe_mfma_bf16", 0, 4000, ctypes.byref(z))
+    L.call("sd3_probe_mfma_bf16", 1, 4000, ctypes.byref(r))
+    assert 250.0 < z.value < 2800.0, z.value
+    assert 250.0 < r.value <= z.value * 1.05, (r.value, z.value)
+    with pytest.raises(L.Sd3Error):
+        L.call("sd3_probe_mfma_bf16", 0, 0, ctypes.byref(z))
+    with pytest.raises(L.Sd3Error):
+        L.call("sd3_probe_mfma_bf16", 0, 100, None)
