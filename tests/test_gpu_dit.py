@@ -83,6 +83,31 @@ def test_dit_bf16_vs_fp32_sd35_medium(side):
     assert rel_l2(run_gpu_dit(k1, "bf16", P)[0], o16[1]) <= 1e-5
 
 
+@pytest.mark.parametrize("B", [1, 4, 8])
+def test_dit_batch_sweep_at_the_benchmark_shape(B):
+    """The 1024x1024 forward at the other batch sizes of the throughput sweep (independent inputs per element): bf16 within
+    relative L2 1e-2 of fp32 on every element, and the last element computed alone equals the same element inside the batch."""
+    cfg = sd35_medium()
+    P = _synthetic_device_params(cfg, 5)
+    k = _inputs(cfg, B, 154, 128, 128, 20 + B)
+    o32 = run_gpu_dit(k, "fp32", P)
+    o16 = run_gpu_dit(k, "bf16", P)
+    assert np.isfinite(o16).all()
+    for b in range(B):
+        assert rel_l2(o16[b], o32[b]) <= BF16_REL_L2, b
+    if B > 1:
+        k1 = dict(k, latent=k["latent"][-1:], captions=k["captions"][-1:], pooled=k["pooled"][-1:], timesteps=k["timesteps"][-1:])
+        assert rel_l2(run_gpu_dit(k1, "bf16", P)[0], o16[-1]) <= 1e-5
+
+
+def test_dit_batch_beyond_the_limit_is_rejected():
+    from sd3_c_amd import lib as L_
+    cfg = DiTConfig(num_layers=1, dual_attention_layers=(), emb_dim=128, attn_heads=2, pooled_dim=64, captions_dim=64, pos_embed_max_size=16, base_height=8)
+    P = _synthetic_device_params(cfg, 3)
+    with pytest.raises(L_.Sd3Error, match="batch"):
+        run_gpu_dit(_inputs(cfg, 9, 2, 8, 8, 4), "bf16", P)
+
+
 def test_dit_ragged_shapes_bf16_vs_fp32():
     """Token counts that are not multiples of any tile (odd grid, 1 text token), reduced depth."""
     cfg = DiTConfig(num_layers=3, dual_attention_layers=(0, 1), emb_dim=512, attn_heads=8, pooled_dim=128, captions_dim=192, pos_embed_max_size=64,
