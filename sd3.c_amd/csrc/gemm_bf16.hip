@@ -95,7 +95,6 @@ __device__ __forceinline__ void gemm_tile(const Prob& pr, const int wg, char* sm
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: LDS destinations of the direct loads are then scalar
     const int wm = wave / WN, wn = wave % WN;
-    const int l32 = lane & 31, lk = lane >> 5;
     int tile_m, tile_n;
     tile_of_workgroup(wg, (M + BM - 1) / BM, (N + BN - 1) / BN, tile_m, tile_n);
     const int m_blk = tile_m * BM, n_blk = tile_n * BN;
@@ -124,98 +123,198 @@ __device__ __forceinline__ void gemm_tile(const Prob& pr, const int wg, char* sm
         for (int i = 0; i < LB; i++) __builtin_amdgcn_global_load_lds((glb_ptr_t)(gb[i] + kt * BK), (lds_ptr_t)(sb + i * NT * 16), 16, 0, 0);
     };
 
-    f32x16_t acc[TM][TN];
+    // Two matrix instructions. 256x256 tiles use v_mfma_f32_16x16x32_bf16: on this device the clock under matrix load is set by
+    // the power limit, and measured on random operands the 16x16x32 form sustains 15-24 % more than 32x32x16 at the same nominal
+    // rate (half as many accumulator updates per product). 128x128 tiles keep v_mfma_f32_32x32x16_bf16: with four wavefronts per
+    // workgroup the finer instruction stream measured 5-15 % slower there. Both forms give bit-identical results.
+    constexpr bool M16 = (BM == 256);
+    constexpr int MI = BM / WM / 16, NJ = BN / WN / 16;      // 16x16 blocks per wavefront
+    f32x16_t acc[M16 ? 1 : TM][M16 ? 1 : TN];
+    f32x4_t acc16[M16 ? MI : 1][M16 ? NJ : 1];
 #pragma unroll
-    for (int i = 0; i < TM; i++)
+    for (int i = 0; i < (M16 ? 1 : TM); i++)
 #pragma unroll
-        for (int j = 0; j < TN; j++)
+        for (int j = 0; j < (M16 ? 1 : TN); j++)
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+#pragma unroll
+    for (int i = 0; i < (M16 ? MI : 1); i++)
+#pragma unroll
+        for (int j = 0; j < (M16 ? NJ : 1); j++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) acc16[i][j][r] = 0.f;
 
     static_assert(STAGES >= 2 && (STAGES - 1) * (LA + LB) < 64, "ring depth: at least two stages, and the loads in flight must fit the 6-bit counter");
     const int nkt = K / BK;
+    const int l32 = lane & 31, lk = lane >> 5;   // position in a 32x32 block
+    const int lr = lane & 15, lg = lane >> 4;    // position in a 16x16 block
 
-    // operand addresses inside a stage: row*128 + ((2*ks + lk) ^ sw)*16 with sw = swz(row) = swz(l32) (block offsets are multiples of 16)
-    const int sw = swz(l32);
-    const int a_off = (wm * (BM / WM) + l32) * 128, b_off = A_BYTES + (wn * (BN / WN) + l32) * 128;
-    // operand fragments of k-step ks live in buffer ks&1; those of step ks+1 are fetched from LDS while the matrix cores work on step ks
-    bf16x8_t a[2][TM], b[2][TN];
-    auto fetch = [&](const char* st, int ks, int buf) {
-        const int ch = ((2 * ks + lk) ^ sw) * 16;
+    if constexpr (M16) {
+        // v_mfma_f32_16x16x32_bf16 operands: lane l holds row (column) l%16 of its block and the 8 consecutive k values 8*(l/16).. of
+        // the 32-deep step: one 16-byte chunk of the row's 128-byte LDS line, chunk (4*step + l/16) ^ swz(row)
+        const int sw = swz(lr);  // (block offsets are multiples of 16 rows, which swz does not see)
+        const int a_off = (wm * (BM / WM) + lr) * 128, b_off = A_BYTES + (wn * (BN / WN) + lr) * 128;
+        // A fragments: one buffer (the fragment of the next step replaces a[i] as soon as row block i is done), except for the last
+        // TAIL row blocks, which have two so that no fragment read is left to issue behind the last matrix instructions of a step
+        // (it would be waited for at once); B fragments: two buffers
+        constexpr int TAIL = MI >= 6 ? 3 : MI / 2, HEAD = MI - TAIL;
+        static_assert(HEAD >= TAIL && TAIL >= 1, "every tail fragment is fetched behind a head row block");
+        bf16x8_t a[HEAD], at[2][TAIL], b[2][NJ];
+        auto a_addr = [&](const char* st, int s, int i) { return reinterpret_cast<const bf16x8_t*>(st + a_off + i * 16 * 128 + (((4 * s + lg) ^ sw) * 16)); };
+        auto load_b = [&](const char* st, int s, int buf) {
 #pragma unroll
-        for (int i = 0; i < TM; i++) a[buf][i] = *reinterpret_cast<const bf16x8_t*>(st + a_off + i * 32 * 128 + ch);
-#pragma unroll
-        for (int j = 0; j < TN; j++) b[buf][j] = *reinterpret_cast<const bf16x8_t*>(st + b_off + j * 32 * 128 + ch);
-    };
-
-    // Every stage is filled up front and exactly one tile is requested per K tile after that (past the end: the last tile
-    // once more, into a buffer nobody reads again), so "tile kt+1 has landed" is always "all but the newest STAGES-2 tiles".
-#pragma unroll
-    for (int s = 0; s < STAGES; s++) issue_tile(min(s, nkt - 1), s);
-    wait_vmcnt<(STAGES - 1) * (LA + LB)>();
-    // tile 0 is in LDS. A bare barrier between compiler fences: __syncthreads() would add a wait for ALL loads in flight
-    asm volatile("" ::: "memory");
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
-    fetch(smem, 0, 0);
-    __builtin_amdgcn_sched_group_barrier(0x100, TM + TN, 0);
-
-    constexpr int KS = BK / 16;
-    // One K tile. The workgroup barrier sits in front of the LAST k-step of a tile, not behind it: by then every fragment
-    // of tile kt is in registers (or on its way: waited for), so its buffer can be handed to the loads of tile kt+2, and the
-    // loads' issue and the first fragment reads of tile kt+1 are interleaved with the matrix instructions of that last
-    // step. With the barrier between tiles instead, the matrix pipeline drains at every tile boundary while all
-    // wavefronts of the compute unit wait for the barrier, issue their loads and wait for their first LDS reads.
-    auto k_tile = [&](const int kt, auto has_next_tag) {
-        constexpr bool HAS_NEXT = decltype(has_next_tag)::value;
-        const char* st = smem + (kt % STAGES) * STAGE_BYTES;
-        auto mfmas = [&](int buf) {
-#pragma unroll
-            for (int i = 0; i < TM; i++)
-#pragma unroll
-                for (int j = 0; j < TN; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[buf][i], b[buf][j], acc[i][j], 0, 0, 0);
+            for (int j = 0; j < NJ; j++) b[buf][j] = *reinterpret_cast<const bf16x8_t*>(st + b_off + j * 16 * 128 + (((4 * s + lg) ^ sw) * 16));
         };
-        // scheduling pattern of a step: behind each of the first matrix instructions one LDS fragment read of the next step
-        // (and, in the last step, one direct global->LDS load of the tile after next), so that their issue and latency are
-        // covered by matrix work
-#pragma unroll
-        for (int ks = 0; ks + 1 < KS; ks++) {
-            fetch(st, ks + 1, (ks + 1) & 1);
-            mfmas(ks & 1);
-#pragma unroll
-            for (int x = 0; x < TM + TN; x++) {
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
-                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // 1 DS read
-            }
-            __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - (TM + TN), 0);
-        }
-        if (HAS_NEXT) {
-            // this thread's loads of tile kt+1 have landed (vmcnt: all but the newest STAGES-2 tiles) and its reads of tile kt are done (lgkmcnt(0))
-            constexpr int INFLIGHT = (STAGES - 2) * (LA + LB);
-            __builtin_amdgcn_s_waitcnt((INFLIGHT & 15) | (7 << 4) | ((INFLIGHT >> 4) << 14));
-            asm volatile("" ::: "memory");  // (the barrier builtin alone does not keep the compiler from moving LDS reads across it)
-            __builtin_amdgcn_s_barrier();
-            asm volatile("" ::: "memory");
-            issue_tile(min(kt + STAGES, nkt - 1), kt % STAGES);
-            fetch(smem + ((kt + 1) % STAGES) * STAGE_BYTES, 0, 0);
-        }
-        mfmas((KS - 1) & 1);
-        if (HAS_NEXT) {
-            constexpr int NLOADS = LA + LB, NM = TM * TN;
-            constexpr int LPS = (NLOADS + NM - 1) / NM;   // loads per slot
-            static_assert(TM + TN <= NM, "more fragment reads than matrix instructions to hide them behind");
-#pragma unroll
-            for (int x = 0; x < NM; x++) {
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                              // 1 MFMA
-                if (x < TM + TN) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);              // 1 DS read
-                if (x * LPS < NLOADS) __builtin_amdgcn_sched_group_barrier(0x020, LPS, 0);       // VMEM reads
-            }
-        }
-    };
-    for (int kt = 0; kt + 1 < nkt; kt++) k_tile(kt, std::true_type{});
-    k_tile(nkt - 1, std::false_type{});
 
-    // ---- epilogue. The MFMA C layout (lane = column, register r = row 8*(r/4) + 4*(lane/32) + r%4) would give 2- or
+        // Every stage is filled up front and exactly one tile is requested per K tile after that (past the end: the last tile
+        // once more, into a buffer nobody reads again), so "tile kt+1 has landed" is always "all but the newest STAGES-2 tiles".
+#pragma unroll
+        for (int s = 0; s < STAGES; s++) issue_tile(min(s, nkt - 1), s);
+        wait_vmcnt<(STAGES - 1) * (LA + LB)>();
+        // tile 0 is in LDS. A bare barrier between compiler fences: __syncthreads() would add a wait for ALL loads in flight
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        load_b(smem, 0, 0);
+#pragma unroll
+        for (int i = 0; i < HEAD; i++) a[i] = *a_addr(smem, 0, i);
+#pragma unroll
+        for (int i = 0; i < TAIL; i++) at[0][i] = *a_addr(smem, 0, HEAD + i);
+        __builtin_amdgcn_sched_group_barrier(0x100, MI + NJ, 0);
+
+        constexpr int KS = BK / 32;
+        static_assert(KS == 2, "two 32-deep steps per K tile");
+        // one 32-deep step on the fragments in a[], at[buf] and b[buf]; with FETCH, the fragments of step ns of stage nst are fetched
+        // behind the matrix instructions: the B fragments first, the A fragment of head row block i once that block is done, the tail
+        // fragments (into the other buffer) behind the first head blocks
+        auto step = [&](int buf, const char* nst, int ns, auto fetch_tag, auto loads_tag) {
+            constexpr bool FETCH = decltype(fetch_tag)::value, LOADS = decltype(loads_tag)::value;
+            constexpr int NLOADS = LA + LB;
+            if (FETCH) load_b(nst, ns, buf ^ 1);
+#pragma unroll
+            for (int i = 0; i < MI; i++) {
+#pragma unroll
+                for (int j = 0; j < NJ; j++) {
+                    acc16[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(i < HEAD ? a[i] : at[buf][i - HEAD], b[buf][j], acc16[i][j], 0, 0, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    if (FETCH && i == 0) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                       // B fragment j of the next step
+                    if (LOADS && i * NJ + j >= NJ && i * NJ + j < NJ + NLOADS) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // one direct load
+                }
+                if (FETCH && i < HEAD) {
+                    a[i] = *a_addr(nst, ns, i);
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                    if (i < TAIL) {
+                        at[buf ^ 1][i] = *a_addr(nst, ns, HEAD + i);
+                        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                    }
+                }
+            }
+        };
+        // One K tile. The workgroup barrier sits in front of the LAST step of a tile, not behind it: by then every fragment
+        // of tile kt is in registers (or on its way: waited for), so its buffer can be handed to the loads of tile kt+STAGES, and the
+        // loads' issue and the fragment reads of tile kt+1 are interleaved with the matrix instructions of that last step.
+        auto k_tile = [&](const int kt, auto has_next_tag) {
+            constexpr bool HAS_NEXT = decltype(has_next_tag)::value;
+            const char* st = smem + (kt % STAGES) * STAGE_BYTES;
+            step(0, st, 1, std::true_type{}, std::false_type{});
+            if (HAS_NEXT) {
+                // this thread's loads of tile kt+1 have landed (vmcnt: all but the newest STAGES-2 tiles) and its reads of tile kt are done (lgkmcnt(0))
+                constexpr int INFLIGHT = (STAGES - 2) * (LA + LB);
+                __builtin_amdgcn_s_waitcnt((INFLIGHT & 15) | (7 << 4) | ((INFLIGHT >> 4) << 14));
+                asm volatile("" ::: "memory");  // (the barrier builtin alone does not keep the compiler from moving LDS reads across it)
+                __builtin_amdgcn_s_barrier();
+                asm volatile("" ::: "memory");
+                issue_tile(min(kt + STAGES, nkt - 1), kt % STAGES);
+                step(1, smem + ((kt + 1) % STAGES) * STAGE_BYTES, 0, std::true_type{}, std::true_type{});
+            } else {
+                step(1, st, 0, std::false_type{}, std::false_type{});
+            }
+        };
+        for (int kt = 0; kt + 1 < nkt; kt++) k_tile(kt, std::true_type{});
+        k_tile(nkt - 1, std::false_type{});
+    } else {
+        // operand addresses inside a stage: row*128 + ((2*ks + lk) ^ sw)*16 with sw = swz(row) = swz(l32) (block offsets are multiples of 16)
+        const int sw = swz(l32);
+        const int a_off = (wm * (BM / WM) + l32) * 128, b_off = A_BYTES + (wn * (BN / WN) + l32) * 128;
+        // operand fragments of k-step ks live in buffer ks&1; those of step ks+1 are fetched from LDS while the matrix cores work on step ks
+        bf16x8_t a[2][TM], b[2][TN];
+        auto fetch = [&](const char* st, int ks, int buf) {
+            const int ch = ((2 * ks + lk) ^ sw) * 16;
+#pragma unroll
+            for (int i = 0; i < TM; i++) a[buf][i] = *reinterpret_cast<const bf16x8_t*>(st + a_off + i * 32 * 128 + ch);
+#pragma unroll
+            for (int j = 0; j < TN; j++) b[buf][j] = *reinterpret_cast<const bf16x8_t*>(st + b_off + j * 32 * 128 + ch);
+        };
+
+        // Every stage is filled up front and exactly one tile is requested per K tile after that (past the end: the last tile
+        // once more, into a buffer nobody reads again), so "tile kt+1 has landed" is always "all but the newest STAGES-2 tiles".
+#pragma unroll
+        for (int s = 0; s < STAGES; s++) issue_tile(min(s, nkt - 1), s);
+        wait_vmcnt<(STAGES - 1) * (LA + LB)>();
+        // tile 0 is in LDS. A bare barrier between compiler fences: __syncthreads() would add a wait for ALL loads in flight
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        fetch(smem, 0, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, TM + TN, 0);
+
+        constexpr int KS = BK / 16;
+        // One K tile. The workgroup barrier sits in front of the LAST k-step of a tile, not behind it: by then every fragment
+        // of tile kt is in registers (or on its way: waited for), so its buffer can be handed to the loads of tile kt+2, and the
+        // loads' issue and the first fragment reads of tile kt+1 are interleaved with the matrix instructions of that last
+        // step. With the barrier between tiles instead, the matrix pipeline drains at every tile boundary while all
+        // wavefronts of the compute unit wait for the barrier, issue their loads and wait for their first LDS reads.
+        auto k_tile = [&](const int kt, auto has_next_tag) {
+            constexpr bool HAS_NEXT = decltype(has_next_tag)::value;
+            const char* st = smem + (kt % STAGES) * STAGE_BYTES;
+            auto mfmas = [&](int buf) {
+#pragma unroll
+                for (int i = 0; i < TM; i++)
+#pragma unroll
+                    for (int j = 0; j < TN; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[buf][i], b[buf][j], acc[i][j], 0, 0, 0);
+            };
+            // scheduling pattern of a step: behind each of the first matrix instructions one LDS fragment read of the next step
+            // (and, in the last step, one direct global->LDS load of the tile after next), so that their issue and latency are
+            // covered by matrix work
+#pragma unroll
+            for (int ks = 0; ks + 1 < KS; ks++) {
+                fetch(st, ks + 1, (ks + 1) & 1);
+                mfmas(ks & 1);
+#pragma unroll
+                for (int x = 0; x < TM + TN; x++) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // 1 DS read
+                }
+                __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - (TM + TN), 0);
+            }
+            if (HAS_NEXT) {
+                // this thread's loads of tile kt+1 have landed (vmcnt: all but the newest STAGES-2 tiles) and its reads of tile kt are done (lgkmcnt(0))
+                constexpr int INFLIGHT = (STAGES - 2) * (LA + LB);
+                __builtin_amdgcn_s_waitcnt((INFLIGHT & 15) | (7 << 4) | ((INFLIGHT >> 4) << 14));
+                asm volatile("" ::: "memory");  // (the barrier builtin alone does not keep the compiler from moving LDS reads across it)
+                __builtin_amdgcn_s_barrier();
+                asm volatile("" ::: "memory");
+                issue_tile(min(kt + STAGES, nkt - 1), kt % STAGES);
+                fetch(smem + ((kt + 1) % STAGES) * STAGE_BYTES, 0, 0);
+            }
+            mfmas((KS - 1) & 1);
+            if (HAS_NEXT) {
+                constexpr int NLOADS = LA + LB, NM = TM * TN;
+                constexpr int LPS = (NLOADS + NM - 1) / NM;   // loads per slot
+                static_assert(TM + TN <= NM, "more fragment reads than matrix instructions to hide them behind");
+#pragma unroll
+                for (int x = 0; x < NM; x++) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                              // 1 MFMA
+                    if (x < TM + TN) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);              // 1 DS read
+                    if (x * LPS < NLOADS) __builtin_amdgcn_sched_group_barrier(0x020, LPS, 0);       // VMEM reads
+                }
+            }
+        };
+        for (int kt = 0; kt + 1 < nkt; kt++) k_tile(kt, std::true_type{});
+        k_tile(nkt - 1, std::false_type{});
+    }
+
+    // ---- epilogue. The MFMA C layouts (32x32: lane = column, register r = row 8*(r/4) + 4*(lane/32) + r%4) would give 2- or
     // 4-byte scattered stores; each wavefront instead transposes one 32-row slab at a time through its private LDS
     // region (the tile ring is free now) and leaves with 16 lanes covering 64 contiguous columns of one row.
     __syncthreads();
@@ -260,10 +359,20 @@ __device__ __forceinline__ void gemm_tile(const Prob& pr, const int wg, char* sm
             for (int p = 0; p < NP; p++) rcur[p] = rnext[p];
             if (i + 1 < TM) request_resid(i + 1);
         }
+        if constexpr (M16) {
+            // C layout of a 16x16 block: lane = column l%16, register r = row 4*(l/16) + r
 #pragma unroll
-        for (int j = 0; j < TN; j++)
+            for (int ii = 0; ii < 2; ii++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) slab[(8 * (r >> 2) + 4 * lk + (r & 3)) * EP + j * 32 + l32] = acc[i][j][r];
+                for (int j = 0; j < NJ; j++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++) slab[(16 * ii + 4 * lg + r) * EP + j * 16 + lr] = acc16[2 * i + ii][j][r];
+        } else {
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) slab[(8 * (r >> 2) + 4 * lk + (r & 3)) * EP + j * 32 + l32] = acc[i][j][r];
+        }
         // LDS operations of one wavefront execute in program order, so the reads below see the writes above without a
         // fence (a fence would also make the wavefront wait for its outstanding global stores on every pass)
         __builtin_amdgcn_wave_barrier();
