@@ -4,7 +4,7 @@ classifier-free-guidance pair), bf16 MFMA path, synthetic inputs and random-init
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--image 1024] [--no-cpu-baseline]
 
 Prints ONE JSON line. A "step" is one full forward. `roofline` describes the kernel class with the largest share of the
-step time, from HIP events recorded around every launch on the library's stream during the timed steps. `cpu_baseline`
+step time, from HIP events recorded around every launch on the library's stream during the timed steps. `power` is the average board power over the timed steps where the machine exposes it. `cpu_baseline`
 times the single-threaded CPU oracle on a bounded sample (one block at full width on few tokens) and converts it with
 the FLOP count of a step; it is a reported baseline, not a target.
 
@@ -79,6 +79,50 @@ def cpu_baseline(cfg, flops_per_step):
                       f"= {rate / 1e9:.3f} GFLOP/s on 1 thread of {os.cpu_count()} visible cores; scaled by FLOP to the {flops_per_step / 1e12:.2f} TFLOP step"}
 
 
+class PowerSampler:
+    """Average board power over a region, from the amdgpu hwmon node (microwatts) if the machine exposes it; None otherwise.
+    The device holds `cap_w` by lowering the clock, which is why the matrix kernels do not reach the published peak."""
+
+    def __init__(self):
+        import glob
+        nodes = sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_input"))
+        self.node = nodes[0] if nodes else None
+        self.samples, self._stop, self._thread = [], False, None
+
+    def _read(self, path):
+        try:
+            with open(path) as f:
+                return int(f.read()) / 1e6
+        except (OSError, ValueError):
+            return None
+
+    def start(self):
+        if not self.node:
+            return
+        import threading
+
+        def run():
+            while not self._stop:
+                w = self._read(self.node)
+                if w is not None:
+                    self.samples.append(w)
+                time.sleep(0.01)
+        self._thread = threading.Thread(target=run, daemon=True)
+        self._thread.start()
+
+    def stop(self, seconds, steps):
+        if not self._thread:
+            return None
+        self._stop = True
+        self._thread.join()
+        if not self.samples:
+            return None
+        avg = sum(self.samples) / len(self.samples)
+        cap = self._read(self.node.replace("power1_input", "power1_cap"))
+        return {"avg_w": round(avg, 1), "max_w": round(max(self.samples), 1), "cap_w": cap, "samples": len(self.samples),
+                "joules_per_step": round(avg * seconds / steps, 2)}
+
+
 def mfma_probe():
     """What this device's matrix cores sustain on the instruction the GEMM and attention kernels use, issued back to back from
     registers by every wavefront (no memory traffic): with zero operands, and with random ones. The device holds its power
@@ -149,11 +193,14 @@ def main():
     for _ in range(a.warmup):
         den(pooled, captions, latent, timesteps, out=out)
     torch.cuda.synchronize()
+    power = PowerSampler()
+    power.start()
     t0 = time.perf_counter()
     for _ in range(a.steps):
         den(pooled, captions, latent, timesteps, out=out)
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
+    power_stats = power.stop(dt, a.steps)
     prof, dt_prof = {}, None
     if not a.no_events:
         den.ctx.profile_begin()
@@ -194,6 +241,7 @@ def main():
         "ms_per_step_profiled": round(dt_prof / a.steps * 1e3, 3) if dt_prof else None,
         "roofline": roofline, "kernels": kernels,
     }
+    res["power"] = power_stats
     if a.precision == "bf16":
         res["mfma_probe"] = mfma_probe()
     if not a.no_cpu_baseline:
