@@ -563,11 +563,11 @@ int gemm_bf16_grouped(const GemmBf16Problem* probs, int n, int out_is_f32, int e
     if (g_gemm_bf16_variant >= 0) return launch(args, m, g_gemm_bf16_variant);
     // Tile shape and grouping by a small cost model. A persistent launch takes ceil(tiles / resident workgroups) rounds; the unit
     // of cost is one round of 256x256 tiles (8 wavefronts, one workgroup per compute unit). Measured on full rounds, a round of
-    // 128x128 tiles (4 wavefronts, two workgroups per unit) takes 0.58 of that for a quarter of the outputs per tile, and a launch
+    // 128x128 tiles (4 wavefronts, two workgroups per unit) takes 0.62 of that for a quarter of the outputs per tile, and a launch
     // of its own for problems with few rows (a short round of small tiles, bound by per-tile overhead) about 0.38.
     const int cus = compute_units();
     if (cus <= 0) return SD3_ERR_HIP;
-    constexpr double ROUND128 = 0.58, SMALL_LAUNCH = 0.38;
+    constexpr double ROUND128 = 0.62, SMALL_LAUNCH = 0.38;
     auto tiles = [](const Prob& q, int t) { return ((q.M + t - 1) / t) * ((q.N + t - 1) / t); };
     auto rounds = [](long long t, int slots) { return (double)((t + slots - 1) / slots); };
     ProbSet big{}, small{};
