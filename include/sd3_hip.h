@@ -121,6 +121,18 @@ int sd3_weights_prepare(sd3_ctx* ctx, int precision);
 int sd3_dit_block(sd3_ctx* ctx, const float* y, float* c, float* x, const char* prefix, int B, int Tc, int Tx, int emb_dim, int attn_heads,
                   int mlp_expand, int use_dual_attention, int use_qk_norm, int discard_context, int precision);
 
+/* No counterpart in the reference. sd3_dit_block for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc): same arguments, same kernels, same results, but the
+ * block's intermediates live in a fixed array of SD3_STATIC_SCRATCH_BYTES that every device the library runs on holds
+ * from load until the process ends, and the call makes no hipMalloc / hipFree / event creation. A block whose
+ * intermediates need more (the size grows with B*(Tc+Tx)*emb_dim) is refused with SD3_ERR_UNSUPPORTED. With SD3_PREC_BF16
+ * the bf16 copies of the block's weights must exist already (one earlier sd3_dit_block call with the same bindings
+ * builds them); otherwise the call returns SD3_ERR_MISSING_PARAM. All calls on one device share the array: calls that
+ * overlap in time on one device (two streams, two contexts, two threads) race. */
+#define SD3_STATIC_SCRATCH_BYTES (64u << 20)
+int sd3_dit_block_static(sd3_ctx* ctx, const float* y, float* c, float* x, const char* prefix, int B, int Tc, int Tx, int emb_dim, int attn_heads,
+                         int mlp_expand, int use_dual_attention, int use_qk_norm, int discard_context, int precision);
+
 /* modules.cpp:1605 DiT_forward(pooled_captions, captions, latent_vector, timesteps, params, num_layers, dual_attention_layers,
  * pooled_dim, captions_dim, C_in, emb_dim, attn_heads, mlp_expand, patch_size, pos_embed_max_size, base_height, use_qk_norm).
  * pooled (B,pooled_dim), captions (B,Tc,captions_dim), latent (B,C_in,H,W), timesteps (B); out (B,C_in,H,W). Inputs are

@@ -33,6 +33,27 @@ const char* last_error() { return g_err; }
 
 using namespace sd3;
 
+// ------------------------------------------------------------------ fixed scratch of the entry point that allocates nothing
+// Lives in device memory from the moment the code object is loaded on a device until the process ends; every device has
+// its own copy at its own address. Host code never uses the array's name as an address: the address on a device is asked
+// for once (static_scratch_of, with that device current) and kept.
+static __device__ __align__(256) unsigned char scratch[SD3_STATIC_SCRATCH_BYTES];
+static constexpr int MAX_DEVICES = 64;
+static void* g_scratch_ptr[MAX_DEVICES] = {};
+
+// the calling thread's current device must be `device`
+static int static_scratch_of(int device, void** out) {
+    if (device < 0 || device >= MAX_DEVICES) return fail(SD3_ERR_UNSUPPORTED, "device %d: at most %d devices", device, MAX_DEVICES);
+    if (!g_scratch_ptr[device]) {
+        void* p = nullptr;
+        SD3_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (!p) return fail(SD3_ERR_HIP, "hipGetSymbolAddress returned a null address for the fixed scratch array on device %d", device);
+        g_scratch_ptr[device] = p;
+    }
+    *out = g_scratch_ptr[device];
+    return SD3_OK;
+}
+
 // ------------------------------------------------------------------ context
 struct PackedWeight {
     void* ptr = nullptr;
@@ -48,6 +69,8 @@ struct sd3_ctx {
     std::map<std::tuple<int, int, int, int, int>, float*> pos_tables;  // (C, max, base, h, w) -> cropped table
     void* ws = nullptr;
     size_t ws_bytes = 0;
+    void* static_scratch = nullptr;  // this device's address of the fixed scratch array (resolved when the context is created)
+    bool no_alloc = false;  // set for the duration of a call that must not allocate: a missing derived weight copy is then an error
     // optional per-kernel-class timing with HIP events on the context's stream
     bool prof_on = false;
     struct ProfSample {
@@ -99,6 +122,10 @@ int get_packed(sd3_ctx* ctx, const float* w, long long K, long long N, int kind,
         *out = it->second.ptr;
         return SD3_OK;
     }
+    if (ctx->no_alloc)
+        return fail(SD3_ERR_MISSING_PARAM,
+                    "the bf16 copy of a %lld x %lld weight has not been built yet and this entry point allocates nothing: run the same block once through "
+                    "sd3_dit_block first (or use SD3_PREC_F32, which reads the bound weights in place)", K, N);
     if (it != ctx->packed.end()) {
         SD3_HIP_TRY(hipStreamSynchronize(ctx->stream));
         SD3_HIP_TRY(hipFree(it->second.ptr));
@@ -134,7 +161,7 @@ struct ProfScope {
     double work;
     long long gemm_launches_before;  // one bracketed call may launch more than one GEMM kernel; the class counts kernels
     ProfScope(sd3_ctx* c, int cls_, double work_) : ctx(c), cls(cls_), work(work_), gemm_launches_before(g_gemm_bf16_launches.load(std::memory_order_relaxed)) {
-        if (!ctx->prof_on) return;
+        if (!ctx->prof_on || ctx->no_alloc) return;  // (creating an event allocates)
         auto get = [&]() -> hipEvent_t {
             hipEvent_t e = nullptr;
             if (!ctx->event_pool.empty()) {
@@ -632,6 +659,15 @@ int sd3_ctx_create(sd3_ctx** out, int device) {
     sd3_ctx* c = new (std::nothrow) sd3_ctx();
     if (!c) return fail(SD3_ERR_OOM, "ctx_create: out of host memory");
     c->device = device;
+    {
+        // the address of the fixed scratch array on this device, asked for once per device with that device current
+        DeviceGuard g(device);
+        int rc = g.ok ? static_scratch_of(device, &c->static_scratch) : fail(SD3_ERR_HIP, "cannot select device %d", device);
+        if (rc != SD3_OK) {
+            delete c;
+            return rc;
+        }
+    }
     *out = c;
     return SD3_OK;
 }
@@ -748,6 +784,32 @@ int sd3_dit_block(sd3_ctx* ctx, const float* y, float* c, float* x, const char* 
     sd3_block_weights w;
     SD3_TRY(lookup_block_weights(ctx, prefix ? prefix : "", d, &w));
     return sd3_dit_block_w(ctx, y, c, x, &w, B, Tc, Tx, emb_dim, attn_heads, mlp_expand, use_dual_attention, use_qk_norm, discard_context, precision);
+}
+
+// The block without any allocation: intermediates live in the fixed scratch array instead of the context's workspace.
+// Calls on one device share that array, so two of them must not overlap in time. Nothing in it has to start at zero:
+// every intermediate is written in full by the kernel that produces it before another kernel reads it.
+int sd3_dit_block_static(sd3_ctx* ctx, const float* y, float* c, float* x, const char* prefix, int B, int Tc, int Tx, int emb_dim, int attn_heads,
+                         int mlp_expand, int use_dual_attention, int use_qk_norm, int discard_context, int precision) {
+    NOTNULL(ctx); NOTNULL(y); NOTNULL(x);
+    SD3_REQUIRE(attn_heads > 0 && emb_dim > 0, "block: emb_dim and attn_heads must be positive");
+    Dims d{B, Tc, Tx, emb_dim, attn_heads, emb_dim / attn_heads, mlp_expand, use_dual_attention != 0, use_qk_norm != 0, discard_context != 0};
+    SD3_TRY(check_block_dims(d, precision));
+    if (Tc > 0) NOTNULL(c);
+    const size_t need = block_workspace_bytes(d, precision);
+    if (need > (size_t)SD3_STATIC_SCRATCH_BYTES)
+        return fail(SD3_ERR_UNSUPPORTED, "dit_block_static: this block needs %zu bytes of intermediates, the fixed scratch array holds %zu; use sd3_dit_block",
+                    need, (size_t)SD3_STATIC_SCRATCH_BYTES);
+    sd3_block_weights w;
+    SD3_TRY(lookup_block_weights(ctx, prefix ? prefix : "", d, &w));
+    DeviceGuard g(ctx->device);
+    if (!g.ok) return fail(SD3_ERR_HIP, "cannot select device %d", ctx->device);
+    if (!ctx->static_scratch) return fail(SD3_ERR_HIP, "dit_block_static: the fixed scratch array has no address on device %d", ctx->device);
+    Bump ws(ctx->static_scratch, SD3_STATIC_SCRATCH_BYTES);
+    ctx->no_alloc = true;
+    const int rc = run_block(ctx, precision, y, c, x, w, d, nullptr, nullptr, ws);
+    ctx->no_alloc = false;
+    return rc;
 }
 
 // ------------------------------------------------------------------ full forward

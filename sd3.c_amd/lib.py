@@ -43,6 +43,7 @@ SIGNATURES = {
     "sd3_weights_clear": [vp],
     "sd3_weights_prepare": [vp, ci],
     "sd3_dit_block": [vp, vp, vp, vp, cs] + [ci] * 10,
+    "sd3_dit_block_static": [vp, vp, vp, vp, cs] + [ci] * 10,
     "sd3_dit_forward": [vp] * 6 + [ci] * 5 + [vp] + [ci] * 12,
     "sd3_dit_forward_cfg_euler": [vp] * 6 + [ci] * 5 + [vp] + [ci] * 12 + [cf, cf],
     "sd3_profile_begin": [vp],

@@ -232,6 +232,15 @@ class Context:
                mlp_expand, int(use_dual_attention), int(use_qk_norm), int(discard_context), _PREC[precision])
         return [c, x]
 
+    def block_static(self, y, c, x, B, Tc, Tx, emb_dim, attn_heads, mlp_expand, use_dual_attention, use_qk_norm, discard_context, precision="fp32",
+                     prefix=""):
+        """`block` without any device allocation: intermediates go to the library's fixed scratch array (64 MiB per device); a block that
+        needs more is refused. With "bf16" the weight copies must exist already (one earlier `block` call builds them)."""
+        L.call("sd3_ctx_set_stream", self._h, _stream())
+        L.call("sd3_dit_block_static", self._h, _p(_dev(y, "y")), _p(_dev(c, "c")), _p(_dev(x, "x")), prefix.encode(), B, Tc, Tx, emb_dim, attn_heads,
+               mlp_expand, int(use_dual_attention), int(use_qk_norm), int(discard_context), _PREC[precision])
+        return [c, x]
+
     def forward(self, pooled_captions, captions, latent_vector, timesteps, num_layers, dual_attention_layers, pooled_dim, captions_dim, C_in, emb_dim,
                 attn_heads, mlp_expand, patch_size, pos_embed_max_size, base_height, use_qk_norm, precision="fp32", out=None):
         lat = _dev(latent_vector, "latent_vector")
