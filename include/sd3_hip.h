@@ -112,8 +112,11 @@ int sd3_ctx_synchronize(sd3_ctx* ctx);
  * valid and unchanged while bound. Names are the reference's (modules.cpp:1558-1575, 1665-1728). */
 int sd3_weights_bind(sd3_ctx* ctx, const char* name, const float* ptr, long long numel);
 int sd3_weights_clear(sd3_ctx* ctx);
-/* Builds (or refreshes) the bf16 MFMA copies of every bound 2-D weight ahead of time. Optional: they are otherwise
- * built on first use. `emb_dim` etc. tell the library which bound tensors are GEMM weights and their shapes. */
+/* Rebuilds, from the current contents of the bound tensors, every derived copy a forward of `precision` uses (bf16: the
+ * K-contiguous bf16 copies of the GEMM weights, the bf16 copies of the adaLN weights and of the patch-conv weight; fp32: the
+ * transposed patch-conv weight). Optional before a first forward (copies are otherwise built on first use, inside that
+ * forward); REQUIRED after changing a bound tensor in place, which the library cannot see. A layer's shape is taken from
+ * its bound `.weight` / `.bias` pair. Re-binding a name with sd3_weights_bind drops the copies of the tensor it replaces. */
 int sd3_weights_prepare(sd3_ctx* ctx, int precision);
 
 /* modules.cpp:1508 DiT_block_forward / modules.cpp:1783 DiT_block_forward_cuda: the block with weights looked up by
@@ -126,8 +129,8 @@ int sd3_dit_block(sd3_ctx* ctx, const float* y, float* c, float* x, const char* 
  * block's intermediates live in a fixed array of SD3_STATIC_SCRATCH_BYTES that every device the library runs on holds
  * from load until the process ends, and the call makes no hipMalloc / hipFree / event creation. A block whose
  * intermediates need more (the size grows with B*(Tc+Tx)*emb_dim) is refused with SD3_ERR_UNSUPPORTED. With SD3_PREC_BF16
- * the bf16 copies of the block's weights must exist already (one earlier sd3_dit_block call with the same bindings
- * builds them); otherwise the call returns SD3_ERR_MISSING_PARAM. All calls on one device share the array: calls that
+ * the bf16 copies of the block's weights must exist already (sd3_weights_prepare, or one earlier sd3_dit_block call with
+ * the same bindings, builds them); otherwise the call returns SD3_ERR_MISSING_PARAM. All calls on one device share the array: calls that
  * overlap in time on one device (two streams, two contexts, two threads) race. */
 #define SD3_STATIC_SCRATCH_BYTES (64u << 20)
 int sd3_dit_block_static(sd3_ctx* ctx, const float* y, float* c, float* x, const char* prefix, int B, int Tc, int Tx, int emb_dim, int attn_heads,
@@ -175,6 +178,32 @@ int sd3_flash_attention_bf16(const void* qkv0, const void* qkv1, void* out0, voi
  * sd3_pack_weight_bf16 into `wpacked`; out bf16. K % 64 == 0 and N % 8 == 0 required. epilogue: 0 bias, 1 bias+GELU-tanh. */
 int sd3_pack_weight_bf16(const float* W, void* wpacked, int K, int N, void* stream);
 int sd3_gemm_bf16(const void* A, const void* wpacked, const float* bias, void* out, int M, int N, int K, int epilogue, void* stream);
+/* The same kernel with every epilogue the block uses and up to three independent problems per launch (in a block: the latent,
+ * dual-branch and context layer of the same kind). epilogue, applied to acc = A @ W (fp32 accumulation):
+ *   0  acc + bias                      (modules.cpp:475-490 linear)
+ *   1  gelu_tanh(acc + bias)           (modules.cpp:1120-1127 mlp, first half)
+ *   2  silu(acc + bias)
+ *   3  resid + gate[m / rows_per_batch] * (acc + bias), fp32, out may equal resid
+ *                                      (linear + gating_mechanism + add, modules.cpp:1435-1436, 1223-1236, 513-518)
+ *   4  acc + bias + table[m % rows_per_batch]      (PatchEmbedding's position table, modules.cpp:1110-1116)
+ *   5  N = 3C packed q|k|v: acc + bias, then per-head RMSNorm (64 columns, eps 1e-6) of the q and k thirds with weights
+ *      rms_q / rms_k (partial_linear x3 + rmsnorm_group x2, modules.cpp:1391-1399)
+ * out is (M, N) row-major, bf16 or (out_is_f32) fp32. Results do not depend on how problems are grouped. */
+typedef struct sd3_gemm_bf16_problem {
+    const void* A;       /* bf16 (M, K) row-major */
+    const void* wpacked; /* from sd3_pack_weight_bf16 */
+    const float* bias;   /* (N) or NULL */
+    void* out;
+    int M, N, K;
+    const float* gate;   /* epilogue 3: (batches, gate_ld) */
+    int gate_ld;
+    const float* resid;  /* epilogue 3: fp32 (M, N) */
+    const float* table;  /* epilogue 4: fp32 (rows_per_batch, N) */
+    int rows_per_batch;  /* epilogues 3 and 4 */
+    const float* rms_q;  /* epilogue 5: 64 floats each, 16-byte aligned */
+    const float* rms_k;
+} sd3_gemm_bf16_problem;
+int sd3_gemm_bf16_grouped(const sd3_gemm_bf16_problem* problems, int n_problems, int epilogue, int out_is_f32, void* stream);
 /* fp32 -> bf16 (round to nearest even) */
 int sd3_cast_f32_to_bf16(const float* in, void* out, long long n, void* stream);
 /* Tuning hook with no counterpart in the reference: forces the output tile of the bf16 GEMM for every later call in this

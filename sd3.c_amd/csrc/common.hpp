@@ -108,7 +108,7 @@ int gemm_f32(const float* A, int lda, const float* W, int ldw, int n0, float* ou
 // bf16 GEMM: A bf16 (M,K) row-major; Wp = packed weight, bf16 (N,K) K-contiguous; out bf16 (out_is_f32 = 0) or fp32.
 int gemm_bf16(const bf16_t* A, const bf16_t* Wp, void* out, int out_is_f32, int ldc, int M, int N, int K, int epi, const GemmEpilogueArgs& ea,
               hipStream_t st);
-// Up to two independent bf16 GEMMs (same epilogue kind and output type) in one launch.
+// Up to three independent bf16 GEMMs (same epilogue kind and output type) in one launch.
 struct GemmBf16Problem {
     const bf16_t* A;
     const bf16_t* Wp;

@@ -64,6 +64,7 @@ struct PackedWeight {
 struct sd3_ctx {
     int device = 0;
     hipStream_t stream = nullptr;
+    hipEvent_t order_event = nullptr;  // orders work across a change of stream (sd3_ctx_set_stream)
     std::unordered_map<std::string, std::pair<const float*, long long>> params;
     std::map<std::pair<const float*, int>, PackedWeight> packed;
     std::map<std::tuple<int, int, int, int, int>, float*> pos_tables;  // (C, max, base, h, w) -> cropped table
@@ -84,6 +85,19 @@ struct sd3_ctx {
 };
 
 namespace {
+
+struct DeviceGuard {
+    int prev = -1;
+    bool ok = false;
+    explicit DeviceGuard(int dev) {
+        if (hipGetDevice(&prev) == hipSuccess && (prev == dev || hipSetDevice(dev) == hipSuccess)) ok = true;
+        else (void)hipGetLastError();
+    }
+    ~DeviceGuard() {
+        int cur = -1;
+        if (ok && hipGetDevice(&cur) == hipSuccess && cur != prev) (void)hipSetDevice(prev);
+    }
+};
 
 struct Bump {
     char* base;
@@ -124,8 +138,8 @@ int get_packed(sd3_ctx* ctx, const float* w, long long K, long long N, int kind,
     }
     if (ctx->no_alloc)
         return fail(SD3_ERR_MISSING_PARAM,
-                    "the bf16 copy of a %lld x %lld weight has not been built yet and this entry point allocates nothing: run the same block once through "
-                    "sd3_dit_block first (or use SD3_PREC_F32, which reads the bound weights in place)", K, N);
+                    "the bf16 copy of a %lld x %lld weight has not been built yet and this entry point allocates nothing: call sd3_weights_prepare "
+                    "(or sd3_dit_block once) first, or use SD3_PREC_F32, which reads the bound weights in place", K, N);
     if (it != ctx->packed.end()) {
         SD3_HIP_TRY(hipStreamSynchronize(ctx->stream));
         SD3_HIP_TRY(hipFree(it->second.ptr));
@@ -149,6 +163,24 @@ int get_packed(sd3_ctx* ctx, const float* w, long long K, long long N, int kind,
     }
     ctx->packed[key] = p;
     *out = p.ptr;
+    return SD3_OK;
+}
+
+// Frees every derived copy made from the tensor at `w` (after the work that may still read them has finished).
+int drop_packed_of(sd3_ctx* ctx, const float* w) {
+    bool synced = false;
+    for (int kind = 0; kind < 3; kind++) {
+        auto it = ctx->packed.find(std::make_pair(w, kind));
+        if (it == ctx->packed.end()) continue;
+        if (!synced) {
+            DeviceGuard g(ctx->device);
+            SD3_HIP_TRY(hipStreamSynchronize(ctx->stream));
+            synced = true;
+        }
+        DeviceGuard g(ctx->device);
+        (void)hipFree(it->second.ptr);
+        ctx->packed.erase(it);
+    }
     return SD3_OK;
 }
 
@@ -475,18 +507,6 @@ int lookup_block_weights(sd3_ctx* ctx, const std::string& prefix, const Dims& d,
     return st;
 }
 
-struct DeviceGuard {
-    int prev = -1;
-    bool ok = false;
-    explicit DeviceGuard(int dev) {
-        if (hipGetDevice(&prev) == hipSuccess && (prev == dev || hipSetDevice(dev) == hipSuccess)) ok = true;
-        else (void)hipGetLastError();
-    }
-    ~DeviceGuard() {
-        int cur = -1;
-        if (ok && hipGetDevice(&cur) == hipSuccess && cur != prev) (void)hipSetDevice(prev);
-    }
-};
 
 }  // namespace
 
@@ -693,6 +713,7 @@ int sd3_ctx_destroy(sd3_ctx* ctx) {
             (void)hipEventDestroy(p.b);
         }
         for (auto e : ctx->event_pool) (void)hipEventDestroy(e);
+        if (ctx->order_event) (void)hipEventDestroy(ctx->order_event);
         (void)hipGetLastError();
     }
     delete ctx;
@@ -700,6 +721,14 @@ int sd3_ctx_destroy(sd3_ctx* ctx) {
 }
 int sd3_ctx_set_stream(sd3_ctx* ctx, void* stream) {
     NOTNULL(ctx);
+    if (ST(stream) == ctx->stream) return SD3_OK;
+    // The workspace, the derived weight copies and the position tables are shared by everything the context enqueues: work
+    // already queued on the old stream must finish before work on the new stream touches them.
+    DeviceGuard g(ctx->device);
+    if (!g.ok) return fail(SD3_ERR_HIP, "cannot select device %d", ctx->device);
+    if (!ctx->order_event) SD3_HIP_TRY(hipEventCreateWithFlags(&ctx->order_event, hipEventDisableTiming));
+    SD3_HIP_TRY(hipEventRecord(ctx->order_event, ctx->stream));
+    SD3_HIP_TRY(hipStreamWaitEvent(ST(stream), ctx->order_event, 0));
     ctx->stream = ST(stream);
     return SD3_OK;
 }
@@ -713,17 +742,48 @@ int sd3_weights_bind(sd3_ctx* ctx, const char* name, const float* ptr, long long
     NOTNULL(ctx); NOTNULL(name); NOTNULL(ptr);
     SD3_REQUIRE(numel > 0, "weights_bind(%s): numel must be positive", name);
     SD3_REQUIRE((reinterpret_cast<uintptr_t>(ptr) & 3) == 0, "weights_bind(%s): pointer is not 4-byte aligned", name);
+    // derived copies are keyed by the tensor's address: what was made from the tensor this name was bound to before, or from
+    // an earlier tensor that lived at the new address, must not survive the re-binding
+    auto old = ctx->params.find(name);
+    if (old != ctx->params.end() && old->second.first != ptr) SD3_TRY(drop_packed_of(ctx, old->second.first));
+    SD3_TRY(drop_packed_of(ctx, ptr));
     ctx->params[name] = std::make_pair(ptr, numel);
     return SD3_OK;
 }
 int sd3_weights_prepare(sd3_ctx* ctx, int precision) {
     NOTNULL(ctx);
     SD3_REQUIRE(precision == SD3_PREC_F32 || precision == SD3_PREC_BF16, "weights_prepare: unknown precision %d", precision);
-    // Drop stale copies; they are rebuilt from the bound fp32 tensors on next use.
     DeviceGuard g(ctx->device);
+    if (!g.ok) return fail(SD3_ERR_HIP, "cannot select device %d", ctx->device);
+    // drop what exists (the bound tensors may have been changed in place) ...
     SD3_HIP_TRY(hipStreamSynchronize(ctx->stream));
     for (auto& kv : ctx->packed) (void)hipFree(kv.second.ptr);
     ctx->packed.clear();
+    // ... and rebuild every copy the forward of this precision would otherwise build on first use. A linear layer's shape follows
+    // from its two bound tensors: `<layer>.bias` has C_out elements and `<layer>.weight` C_in * C_out.
+    auto ends_with = [](const std::string& s, const char* suffix) {
+        const size_t n = std::strlen(suffix);
+        return s.size() >= n && s.compare(s.size() - n, n, suffix) == 0;
+    };
+    for (auto& kv : ctx->params) {
+        const std::string& name = kv.first;
+        if (!ends_with(name, ".weight")) continue;
+        auto b = ctx->params.find(name.substr(0, name.size() - 6) + "bias");
+        if (b == ctx->params.end() || b->second.second <= 0 || kv.second.second % b->second.second) continue;
+        const long long N = b->second.second, K = kv.second.second / N;
+        const void* unused = nullptr;
+        if (name == "to_patch.conv.weight") {  // (C_out, C_in*p*p): bf16 cast for the MFMA GEMM, fp32 transpose for the fp32 one
+            if (precision == SD3_PREC_BF16) SD3_TRY(get_packed(ctx, kv.second.first, N, K, 1, &unused));
+            else SD3_TRY(get_packed(ctx, kv.second.first, K, N, 2, &unused));
+            continue;
+        }
+        if (precision != SD3_PREC_BF16) continue;
+        const bool adaln = ends_with(name, "ada_lnorm.linear.weight") || name == "ada_ln_out.linear.weight";
+        const bool gemm = ends_with(name, "_to_qkv.weight") || ends_with(name, "_attn_Wout.weight") || ends_with(name, "_mlp.lin1.weight") ||
+                          ends_with(name, "_mlp.lin2.weight") || name == "captions_linear.weight" || name == "linear_out.weight";
+        if (adaln) SD3_TRY(get_packed(ctx, kv.second.first, K, N, 1, &unused));
+        else if (gemm && K % 64 == 0) SD3_TRY(get_packed(ctx, kv.second.first, K, N, 0, &unused));
+    }
     return SD3_OK;
 }
 
@@ -1040,6 +1100,32 @@ int sd3_gemm_bf16(const void* A, const void* wpacked, const float* bias, void* o
     GemmEpilogueArgs ea;
     ea.bias = bias;
     return gemm_bf16((const bf16_t*)A, (const bf16_t*)wpacked, out, 0, N, M, N, K, epilogue, ea, ST(stream));
+}
+int sd3_gemm_bf16_grouped(const sd3_gemm_bf16_problem* problems, int n_problems, int epilogue, int out_is_f32, void* stream) {
+    NOTNULL(problems);
+    SD3_REQUIRE(n_problems >= 1 && n_problems <= 3, "gemm_bf16_grouped: 1 to 3 problems per launch (got %d)", n_problems);
+    SD3_REQUIRE(epilogue >= EPI_BIAS && epilogue <= EPI_QKV_NORM, "gemm_bf16_grouped: unknown epilogue %d", epilogue);
+    GemmBf16Problem probs[3];
+    for (int i = 0; i < n_problems; i++) {
+        const sd3_gemm_bf16_problem& q = problems[i];
+        SD3_REQUIRE(q.M >= 0 && q.N > 0 && q.K > 0, "gemm_bf16_grouped: bad sizes in problem %d (M=%d N=%d K=%d)", i, q.M, q.N, q.K);
+        if (q.M > 0) SD3_REQUIRE(q.A && q.wpacked && q.out, "gemm_bf16_grouped: null operand in problem %d", i);
+        GemmEpilogueArgs ea;
+        ea.bias = q.bias;
+        ea.rows_per_batch = q.rows_per_batch > 0 ? q.rows_per_batch : 1;
+        if (epilogue == EPI_GATE_RESID) {
+            if (q.M > 0) SD3_REQUIRE(q.gate && q.resid && q.gate_ld >= q.N, "gemm_bf16_grouped: the gated epilogue needs gate (row stride >= N) and resid in problem %d", i);
+            SD3_REQUIRE(out_is_f32, "gemm_bf16_grouped: the gated epilogue updates an fp32 residual stream (out_is_f32 must be 1)");
+            ea.gate = q.gate; ea.gate_ld = q.gate_ld; ea.resid = q.resid;
+        } else if (epilogue == EPI_BIAS_ROWADD) {
+            if (q.M > 0) SD3_REQUIRE(q.table, "gemm_bf16_grouped: the row-table epilogue needs a table in problem %d", i);
+            ea.table = q.table;
+        } else if (epilogue == EPI_QKV_NORM) {
+            ea.gate = q.rms_q; ea.resid = q.rms_k;  // (checked by the launcher: both present, 16-byte aligned, N = 3C with C % 64 == 0)
+        }
+        probs[i] = GemmBf16Problem{(const bf16_t*)q.A, (const bf16_t*)q.wpacked, q.out, q.N, q.M, q.N, q.K, ea};
+    }
+    return gemm_bf16_grouped(probs, n_problems, out_is_f32, epilogue, ST(stream));
 }
 int sd3_cast_f32_to_bf16(const float* in, void* out, long long n, void* stream) {
     SD3_REQUIRE(n >= 0, "cast: negative size");

@@ -457,7 +457,7 @@ __device__ __forceinline__ void gemm_tile(const Prob& pr, const int wg, char* sm
     }
 }
 
-// Persistent kernel: one workgroup per compute unit walks over the tiles of up to two problems. The stores of a finished
+// Persistent kernel: one workgroup per compute unit walks over the tiles of up to three problems. The stores of a finished
 // tile drain while the next tile's K loop is already running, instead of holding the compute unit until they retire.
 // Workgroup g takes work items g, g + G, g + 2G ... (G = grid size, a multiple of 8), so it stays on its XCD's run of tiles.
 template <int BM, int BN, int WM, int WN, int STAGES, int EPI, bool OUT_F32>

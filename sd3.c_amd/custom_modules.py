@@ -6,8 +6,9 @@ points only, so that scripts written like the reference's drivers run against th
                   in_channels, emb_dim, attn_heads, mlp_expand, patch_size, pos_embed_max_size, base_height, use_qk_norm)
 
 The reference's `Dit_block` and `DiT` take host tensors and compute on the CPU (module_tests/DiT.py:33-47,
-module_tests/dit_block.py:40-46); here the same calls copy their arguments to the GPU, run the fp32 path (the one held to
-the reference's 1e-4 / 1e-5 comparisons) and copy the results back, keeping the in-place contract of the block:
+module_tests/dit_block.py:40-46); here the same calls copy their arguments to the GPU, run the path named by the module-level
+`PRECISION` ("fp32", the default: the one held to the reference's 1e-4 / 1e-5 comparisons; set `F.PRECISION = "bf16"` for the
+bf16 MFMA throughput path, relative L2 <= 1e-2) and copy the results back, keeping the in-place contract of the block:
 `context_embeddings` and `latent_vector` are overwritten and returned. `DiT_block_cuda` takes device tensors as in
 module_tests/dit_block.py:60-66. There is no CPU fallback: without a GPU every call raises.
 
@@ -29,6 +30,7 @@ if "sd3_c_amd" not in sys.modules:  # the package directory name has a dot in it
 from sd3_c_amd import modules as _M  # noqa: E402
 
 _DEV = "cuda"
+PRECISION = "fp32"  # "fp32" | "bf16": the arithmetic of Dit_block / DiT_block_cuda / DiT (the reference's signatures have no slot for it)
 
 
 def _up(t):
@@ -76,7 +78,7 @@ def Dit_block(temp_embeddings, context_embeddings, latent_vector, params, B, Tc,
     """modules.cpp:1508 DiT_block_forward on host tensors: context_embeddings and latent_vector are updated in place and returned."""
     y, c, x = _up(temp_embeddings), _up(context_embeddings), _up(latent_vector)
     c, x = _M.Dit_block(y, c, x, _params_up(params), B, Tc, Tx, emb_dim, attn_heads, mlp_expand, use_dual_attention, use_qk_norm, discard_context,
-                        precision="fp32")
+                        precision=PRECISION)
     context_embeddings.copy_(c.to(context_embeddings.device))
     latent_vector.copy_(x.to(latent_vector.device))
     return [context_embeddings, latent_vector]
@@ -86,7 +88,7 @@ def DiT_block_cuda(temp_embeddings, context_embeddings, latent_vector, params, B
                    use_qk_norm, discard_context):
     """modules.cpp:1783 DiT_block_forward_cuda: device tensors, updated in place and returned."""
     return _M.Dit_block(temp_embeddings, context_embeddings, latent_vector, params, B, Tc, Tx, emb_dim, attn_heads, mlp_expand, use_dual_attention,
-                        use_qk_norm, discard_context, precision="fp32")
+                        use_qk_norm, discard_context, precision=PRECISION)
 
 
 def DiT(pooled_captions, captions, latent_vector, timesteps, params, num_layers, dual_attention_layers, pooled_dim, captions_dim, C_in, emb_dim, attn_heads,
@@ -94,5 +96,5 @@ def DiT(pooled_captions, captions, latent_vector, timesteps, params, num_layers,
     """modules.cpp:1605 DiT_forward on host (or device) tensors: returns a new (B, C_in, H, W) tensor on the latent's device."""
     out = _M.DiT(_up(pooled_captions), _up(captions), _up(latent_vector), _up(timesteps), _params_up(params), num_layers, dual_attention_layers,
                  pooled_dim, captions_dim, C_in, emb_dim, attn_heads, mlp_expand, patch_size, pos_embed_max_size, base_height, use_qk_norm,
-                 precision="fp32")
+                 precision=PRECISION)
     return out.to(latent_vector.device)

@@ -51,10 +51,17 @@ SIGNATURES = {
     "sd3_flash_attention_bf16": [vp] * 8 + [ci] * 5 + [vp],
     "sd3_pack_weight_bf16": [vp, vp, ci, ci, vp],
     "sd3_gemm_bf16": [vp, vp, vp, vp, ci, ci, ci, ci, vp],
+    "sd3_gemm_bf16_grouped": [vp, ci, ci, ci, vp],
     "sd3_cast_f32_to_bf16": [vp, vp, cll, vp],
     "sd3_gemm_bf16_force_tile": [ci],
     "sd3_probe_mfma_bf16": [ci, ci, vp],
 }
+
+
+class GemmBf16Problem(C.Structure):
+    """sd3_gemm_bf16_problem of include/sd3_hip.h"""
+    _fields_ = [("A", vp), ("wpacked", vp), ("bias", vp), ("out", vp), ("M", ci), ("N", ci), ("K", ci), ("gate", vp), ("gate_ld", ci), ("resid", vp),
+                ("table", vp), ("rows_per_batch", ci), ("rms_q", vp), ("rms_k", vp)]
 
 
 class Sd3Error(RuntimeError):

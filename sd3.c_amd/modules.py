@@ -78,6 +78,16 @@ def silu(input):
     return y
 
 
+def add(input, other):
+    """modules.cpp:513 add: element-wise sum (the residual adds of the block, modules.cpp:1462, 1485-1486)."""
+    a, b = _dev(input, "input"), _dev(other, "other")
+    if a.shape != b.shape:
+        raise ValueError("add: shapes differ")
+    out = torch.empty_like(a)
+    L.call("sd3_add", _p(a), _p(b), _p(out), a.numel(), _stream())
+    return out
+
+
 def linear(input, weight, bias):
     """modules.cpp:538 Linear_forward: weight is (C_in, C_out)."""
     x, W, b = _dev(input, "input"), _dev(weight, "weight"), _dev(bias, "bias")

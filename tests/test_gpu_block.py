@@ -64,6 +64,78 @@ def test_block_fp32_width_1536_vs_oracle(dual, discard):
     co, xo = ol.orc_dit_block(k["y"], k["c"], k["x"], k["params"], 24, 4, dual, True, discard)
     assert max_abs(x, xo) <= F32_TOL
     assert max_abs(c, co) <= F32_TOL
+    # the bf16 path against the CPU arithmetic directly (not through the fp32 GPU path)
+    c16, x16 = run_gpu_block(k, "bf16")
+    assert rel_l2(x16, xo) <= BF16_REL_L2 and rel_l2(x16 - k["x"], xo - k["x"]) <= 2 * BF16_REL_L2
+    if not discard:
+        assert rel_l2(c16, co) <= BF16_REL_L2
+
+
+@pytest.mark.parametrize("name", [n for n in cases.BLOCK_CASES if n.endswith("hs64")])
+def test_block_bf16_vs_reference_golden(name):
+    """The bf16 path against the outputs of the compiled reference (head_dim 64 cases; weights N(0, 0.1), so the block's update is as
+    large as the stream it is added to)."""
+    k = cases.block_case(name)
+    c, x = run_gpu_block(k, "bf16")
+    assert rel_l2(x, GOLDEN[name + ".x"]) <= BF16_REL_L2
+    if k["discard_context"]:
+        assert np.array_equal(c, k["c"])
+    else:
+        assert rel_l2(c, GOLDEN[name + ".c"]) <= BF16_REL_L2
+
+
+@pytest.mark.parametrize("precision", ["fp32", "bf16"])
+def test_rebinding_a_name_or_refreshing_drops_the_derived_weight_copies(precision):
+    """Derived copies (bf16 GEMM / adaLN weights) are keyed by the bound tensor's address: binding new contents at the same address, or
+    changing a bound tensor in place and calling refresh(), must be seen by the next call."""
+    k = cases.block_case("block_dual_hs64")
+    B, Tc, Cd = k["c"].shape
+    Tx = k["x"].shape[1]
+    args = (B, Tc, Tx, Cd, k["NH"], k["mlp_expand"], True, True, False)
+
+    def fresh(params):
+        c, x = M.Dit_block(dev(k["y"]), dev(k["c"]), dev(k["x"]), dev_params(params), *args, precision=precision)
+        return host(c), host(x)
+
+    P2 = dict(k["params"])
+    for n in ("latent_mlp.lin2.weight", "latent_ada_lnorm.linear.weight", "context_to_qkv.weight"):
+        P2[n] = np.ascontiguousarray(P2[n][::-1] * 1.5)
+    want1, want2 = fresh(k["params"]), fresh(P2)
+    assert not np.array_equal(want1[1], want2[1])
+    ctx = M.Context()
+    try:
+        dP = dev_params(k["params"])
+        ctx.bind(dP)
+        run = lambda: tuple(host(t) for t in ctx.block(dev(k["y"]), dev(k["c"]), dev(k["x"]), *args, precision=precision))  # noqa: E731
+        got = run()
+        assert np.array_equal(got[1], want1[1]) and np.array_equal(got[0], want1[0])
+        for n in ("latent_mlp.lin2.weight", "latent_ada_lnorm.linear.weight"):   # new contents at the same address, bound again
+            dP[n].copy_(dev(P2[n]))
+            ctx.bind({n: dP[n]})
+        dP["context_to_qkv.weight"].copy_(dev(P2["context_to_qkv.weight"]))      # changed in place without re-binding: refresh()
+        ctx.refresh(precision)
+        got = run()
+        assert np.array_equal(got[1], want2[1]) and np.array_equal(got[0], want2[0])
+    finally:
+        ctx.close()
+
+
+def test_prepare_builds_the_bf16_copies_ahead_of_the_first_call():
+    """After refresh() the first bf16 call finds every copy: shown with the entry point that refuses to allocate."""
+    k = cases.block_case("block_dual_hs64")
+    B, Tc, Cd = k["c"].shape
+    Tx = k["x"].shape[1]
+    args = (B, Tc, Tx, Cd, k["NH"], k["mlp_expand"], True, True, False)
+    ctx = M.Context()
+    try:
+        ctx.bind(dev_params(k["params"]))
+        ctx.refresh("bf16")
+        c, x = ctx.block_static(dev(k["y"]), dev(k["c"]), dev(k["x"]), *args, precision="bf16")
+        c2, x2 = ctx.block(dev(k["y"]), dev(k["c"]), dev(k["x"]), *args, precision="bf16")
+        assert torch.equal(x, x2) and torch.equal(c, c2)
+        assert rel_l2(host(x), GOLDEN["block_dual_hs64.x"]) <= BF16_REL_L2
+    finally:
+        ctx.close()
 
 
 @pytest.mark.parametrize("dual", [True, False])

@@ -50,6 +50,23 @@ def test_block_called_like_module_tests_dit_block_py(name):
     assert x2 is xd and torch.equal(xd.cpu(), x)
 
 
+def test_module_level_precision_switch_reaches_the_bf16_path():
+    """A script written against the reference's signatures selects the bf16 path with F.PRECISION; results then differ from the
+    fp32 ones in the low bits only (and the switch goes back)."""
+    from gpu_util import rel_l2
+    k = cases.block_case("block_dual_hs64")
+    (B, Tc, C), Tx = k["c"].shape, k["x"].shape[1]
+    params = {n: torch.from_numpy(v) for n, v in k["params"].items()}
+    try:
+        F.PRECISION = "bf16"
+        y, c, x = torch.from_numpy(k["y"].copy()), torch.from_numpy(k["c"].copy()), torch.from_numpy(k["x"].copy())
+        F.Dit_block(y, c, x, params, B, Tc, Tx, C, k["NH"], k["mlp_expand"], k["use_dual"], k["use_qk_norm"], k["discard_context"])
+    finally:
+        F.PRECISION = "fp32"
+    gold = GOLDEN["block_dual_hs64.x"]
+    assert 1e-6 < rel_l2(x.numpy(), gold) <= 1e-2
+
+
 def test_operator_entry_points_take_host_tensors():
     x = torch.randn(2, 5, 64)
     out = F.layer_norm(x, None, None, 1e-6, False)[0]

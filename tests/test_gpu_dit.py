@@ -46,6 +46,46 @@ def test_dit_fp32_reference_test_configuration():
     assert max_abs(run_gpu_dit(k), gold) <= F32_TOL
 
 
+def test_dit_bf16_vs_reference_golden():
+    """The bf16 path against the output of the compiled reference directly (the one golden forward whose sizes suit the bf16
+    kernels: heads of 64, every width a multiple of 64)."""
+    k = cases.dit_case("dit_hs64")
+    out = run_gpu_dit(k, "bf16")
+    assert rel_l2(out, GOLDEN["dit_hs64.out"]) <= BF16_REL_L2
+
+
+@pytest.mark.parametrize("file_dtype,shards", [("float32", 1), ("bfloat16", 3)])
+def test_dit_from_hugging_face_safetensors_vs_reference_golden(tmp_path, file_dtype, shards):
+    """Real-weight path end to end: the parameters of the reference's own full-model test configuration written the way the Hugging
+    Face checkpoint stores them (its names, nn.Linear layout, separate q/k/v; module_tests/modules.py:532-612), as one fp32 file or
+    as bf16 shards with an index -> load_safetensors -> Denoiser on the GPU -> the compiled reference's output."""
+    import json
+    from safetensors.torch import save_file
+    from sd3_c_amd import hf_weights as H
+    k = cases.dit_reference_test_case()
+    cfg = k["cfg"]
+    hf = {n: torch.from_numpy(v).to(getattr(torch, file_dtype)) for n, v in H.to_hf_state_dict(k["params"], cfg).items()}
+    names = sorted(hf)
+    weight_map = {}
+    for i in range(shards):
+        fn = f"diffusion_pytorch_model-{i + 1:05d}-of-{shards:05d}.safetensors" if shards > 1 else "diffusion_pytorch_model.safetensors"
+        part = {n: hf[n].contiguous() for n in names[i::shards]}
+        save_file(part, str(tmp_path / fn))
+        weight_map.update({n: fn for n in part})
+    if shards > 1:
+        (tmp_path / "diffusion_pytorch_model.safetensors.index.json").write_text(json.dumps({"metadata": {}, "weight_map": weight_map}))
+    loaded = H.load_safetensors(str(tmp_path), cfg)
+    assert list(loaded) == list(k["params"])
+    gold = np.load(os.path.join(HERE, "golden", "reference_dit_test_config.npz"))["out"]
+    den = M.Denoiser(dev_params(loaded), cfg, "fp32")
+    out = host(den(dev(k["pooled"]), dev(k["captions"]), dev(k["latent"]), dev(k["timesteps"])))
+    if file_dtype == "float32":
+        assert max_abs(out, gold) <= F32_TOL          # lossless file: the fp32 parity bar
+    else:
+        assert rel_l2(out, gold) <= BF16_REL_L2       # weights rounded to bf16 in the file: the bf16 bar
+    den.ctx.close()
+
+
 def _synthetic_device_params(cfg, seed):
     g = torch.Generator(device="cuda").manual_seed(seed)
     P = {}

@@ -143,6 +143,19 @@ def test_modulation_gating_concat_split():
     assert np.array_equal(host(s1), a) and np.array_equal(host(s2), b)
 
 
+@pytest.mark.parametrize("n", [1, 3, 4, 1000, 4099, 1 << 20])
+def test_add(n):
+    """modules.cpp:513-518; sizes around the vector width of the kernel; in place on the first operand as the block uses it."""
+    a, b = randn(n) * 3, randn(n) * 1e-3
+    ref = np.empty_like(a)
+    ol.oracle().orc_add(fp(a), fp(b), fp(ref), C.c_long(n))
+    assert np.array_equal(host(M.add(dev(a), dev(b))), ref)
+    da = dev(a)
+    from sd3_c_amd import lib as L_
+    L_.call("sd3_add", da.data_ptr(), dev(b).data_ptr(), da.data_ptr(), n, None)
+    assert np.array_equal(host(da), ref)
+
+
 def test_empty_and_invalid_inputs():
     from sd3_c_amd import lib as L_
     e = torch.empty((0, 4, 8), device="cuda")
