@@ -49,6 +49,22 @@ def test_reference_named_cpp_overloads_compile():
     assert r.returncode == 0, r.stderr
 
 
+def test_cpp_callers_of_the_boundary_are_built_and_link():
+    """tests/cpp: the C++ program over modules_api.hpp and the reference-side torch binding (run on the GPU by
+    tests/test_gpu_cpp_boundary.py); here: they exist, resolve their libraries, and the binding imports and exports its two entry points."""
+    import sys
+    cpp = os.path.join(ROOT, "tests", "cpp")
+    if not (os.path.exists(os.path.join(cpp, "host_block")) and os.path.exists(os.path.join(cpp, "sd3_ref_binding.so"))):
+        r = subprocess.run(["make", "-C", cpp], capture_output=True, text=True)
+        assert r.returncode == 0, r.stderr[-2000:]
+    r = subprocess.run(["ldd", os.path.join(cpp, "host_block")], capture_output=True, text=True)
+    assert "libsd3_hip.so =>" in r.stdout and "not found" not in r.stdout, r.stdout
+    import torch  # noqa: F401  (the binding links against torch's libraries)
+    sys.path.insert(0, cpp)
+    import sd3_ref_binding
+    assert callable(sd3_ref_binding.DiT_block_cuda) and callable(sd3_ref_binding.DiT_cuda)
+
+
 def test_argument_errors_are_status_codes_not_exits():
     lib = L.load()
     assert lib.sd3_version() >= 1
