@@ -192,7 +192,9 @@ struct ProfScope {
     int cls;
     double work;
     long long gemm_launches_before;  // one bracketed call may launch more than one GEMM kernel; the class counts kernels
-    ProfScope(sd3_ctx* c, int cls_, double work_) : ctx(c), cls(cls_), work(work_), gemm_launches_before(g_gemm_bf16_launches.load(std::memory_order_relaxed)) {
+    long long explicit_launches;     // kernels launched inside the bracket when the caller knows the number (0: count GEMM kernels, at least 1)
+    ProfScope(sd3_ctx* c, int cls_, double work_, long long launches_ = 0)
+        : ctx(c), cls(cls_), work(work_), gemm_launches_before(g_gemm_bf16_launches.load(std::memory_order_relaxed)), explicit_launches(launches_) {
         if (!ctx->prof_on || ctx->no_alloc) return;  // (creating an event allocates)
         auto get = [&]() -> hipEvent_t {
             hipEvent_t e = nullptr;
@@ -213,7 +215,7 @@ struct ProfScope {
         if (!a || !b) return;
         (void)hipEventRecord(b, ctx->stream);
         const long long kernels = g_gemm_bf16_launches.load(std::memory_order_relaxed) - gemm_launches_before;
-        ctx->prof.push_back({a, b, cls, work, kernels > 1 ? kernels : 1});
+        ctx->prof.push_back({a, b, cls, work, explicit_launches > 0 ? explicit_launches : (kernels > 1 ? kernels : 1)});
     }
 };
 
@@ -299,7 +301,7 @@ int ada_jobs_run(sd3_ctx* ctx, int prec, const float* y, int B, int C, std::vect
     }
     double bytes = 0;
     for (auto& j : jobs) bytes += (double)C * j.N * (prec == SD3_PREC_BF16 ? 2 : 4) + (double)B * j.N * 4;
-    ProfScope ps(ctx, SD3_PROF_ADALN, bytes);
+    ProfScope ps(ctx, SD3_PROF_ADALN, bytes, ((long long)jobs.size() + 15) / 16);  // one kernel per 16 weight matrices
     return small_linear_batched(y, B, C, jobs.data(), (int)jobs.size(), prec == SD3_PREC_BF16, -1, ctx->stream);
 }
 

@@ -90,7 +90,7 @@ __device__ __forceinline__ void gemm_tile(const Prob& pr, const int wg, char* sm
     constexpr int A_BYTES = BM * 128, STAGE_BYTES = (BM + BN) * 128;
     constexpr int LA = BM * 8 / NT, LB = BN * 8 / NT;        // 16-byte chunks per thread per tile
     static_assert(BM * 8 % NT == 0 && BN * 8 % NT == 0, "tile rows must divide evenly over the threads");
-    static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0, "wavefront tiles are made of 32x32 blocks");
+    static_assert(BM % (WM * 16) == 0 && BN % (WN * 16) == 0 && (BM == 256 || (BM % (WM * 32) == 0 && BN % (WN * 32) == 0)), "wavefront tiles are made of 16x16 (256-row tiles) or 32x32 blocks");
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: LDS destinations of the direct loads are then scalar
@@ -321,15 +321,23 @@ __device__ __forceinline__ void gemm_tile(const Prob& pr, const int wg, char* sm
     constexpr int WNC = BN / WN;        // columns per wavefront
     constexpr int EP = WNC + 4;         // fp32 pitch of the staging slab
     static_assert(WM * WN * 32 * EP * 4 <= smem_bytes<BM, BN, WM, WN, STAGES>(), "epilogue staging must fit in the LDS allocation");
+    constexpr int CPR = WNC / 4;        // float4 chunks per row
+    static_assert(WNC % 4 == 0 && CPR <= 64, "a row of the wavefront's slab is made of float4 chunks");
+    // rows covered by one pass of the wavefront: the largest power of two with RPI * CPR <= 64 (when CPR does not divide 64, as with
+    // 48-column slabs, the lanes beyond RPI * CPR sit the epilogue out)
+    constexpr int RPI = CPR > 32 ? 1 : CPR > 16 ? 2 : CPR > 8 ? 4 : CPR > 4 ? 8 : CPR > 2 ? 16 : 32;
+    // rows per slab: 32, or 16 where 32 would take more than four passes (the row registers of a slab are all live at once)
+    constexpr int SR = (M16 && 32 / RPI > 4) ? 16 : 32;
+    constexpr int NSLAB = BM / WM / SR;
+    constexpr int NP = SR / RPI;        // rows of a slab per lane
     float* slab = reinterpret_cast<float*>(smem) + wave * 32 * EP;
     float* outf = reinterpret_cast<float*>(out_);
     bf16_t* outh = reinterpret_cast<bf16_t*>(out_);
-    constexpr int CPR = WNC / 4;        // float4 chunks per row
-    constexpr int RPI = 64 / CPR;       // rows covered by one pass of the wavefront
-    const int e_row = lane / CPR, e_col = (lane % CPR) * 4;
+    const bool lane_on = lane < RPI * CPR;
+    const int e_row = lane_on ? lane / CPR : 0, e_col = lane_on ? (lane % CPR) * 4 : 0;
     const int n0 = n_blk + wn * WNC + e_col;
     const bool vec_ok = ((N & 3) == 0) && ((ldc & 3) == 0);
-    const int nvalid = min(4, N - n0);  // <= 0 for lanes beyond the last column
+    const int nvalid = lane_on ? min(4, N - n0) : 0;  // <= 0 for lanes beyond the last column (and for lanes that sit out)
     float bias4[4] = {0.f, 0.f, 0.f, 0.f};
     if (epi.bias)
 #pragma unroll
@@ -337,7 +345,6 @@ __device__ __forceinline__ void gemm_tile(const Prob& pr, const int wg, char* sm
             if (c < nvalid) bias4[c] = epi.bias[n0 + c];
     // batch index of a row without a division per row: the tile starts in batch b0 and crosses a boundary every rpb rows
     const int rpb = epi.rows_per_batch, b0 = m_blk / rpb;
-    constexpr int NP = 32 / RPI;        // rows of a slab per lane
     // gated layers: the residual rows of the NEXT slab are requested before the current slab goes through LDS, so that
     // their latency is not paid once per slab with nothing else to do
     constexpr bool PREFETCH_RESID = (EPI == EPI_GATE_RESID);
@@ -346,27 +353,27 @@ __device__ __forceinline__ void gemm_tile(const Prob& pr, const int wg, char* sm
         if (PREFETCH_RESID && vec_ok)
 #pragma unroll
             for (int p = 0; p < NP; p++) {
-                const int m = m_blk + wm * (BM / WM) + i * 32 + p * RPI + e_row;
+                const int m = m_blk + wm * (BM / WM) + i * SR + p * RPI + e_row;
                 if (m < M && nvalid > 0) rnext[p] = *reinterpret_cast<const float4*>(epi.resid + (long long)m * ldc + n0);
             }
     };
     request_resid(0);
 #pragma unroll
-    for (int i = 0; i < TM; i++) {
+    for (int i = 0; i < NSLAB; i++) {
         float4 rcur[PREFETCH_RESID ? NP : 1];
         if (PREFETCH_RESID) {
 #pragma unroll
             for (int p = 0; p < NP; p++) rcur[p] = rnext[p];
-            if (i + 1 < TM) request_resid(i + 1);
+            if (i + 1 < NSLAB) request_resid(i + 1);
         }
         if constexpr (M16) {
             // C layout of a 16x16 block: lane = column l%16, register r = row 4*(l/16) + r
 #pragma unroll
-            for (int ii = 0; ii < 2; ii++)
+            for (int ii = 0; ii < SR / 16; ii++)
 #pragma unroll
                 for (int j = 0; j < NJ; j++)
 #pragma unroll
-                    for (int r = 0; r < 4; r++) slab[(16 * ii + 4 * lg + r) * EP + j * 16 + lr] = acc16[2 * i + ii][j][r];
+                    for (int r = 0; r < 4; r++) slab[(16 * ii + 4 * lg + r) * EP + j * 16 + lr] = acc16[(SR / 16) * i + ii][j][r];
         } else {
 #pragma unroll
             for (int j = 0; j < TN; j++)
@@ -385,7 +392,7 @@ __device__ __forceinline__ void gemm_tile(const Prob& pr, const int wg, char* sm
 #pragma unroll
         for (int p = 0; p < NP; p++) {
             const int row = p * RPI + e_row;
-            const int m = m_blk + wm * (BM / WM) + i * 32 + row;
+            const int m = m_blk + wm * (BM / WM) + i * SR + row;
             if (m < M && nvalid > 0) {
                 const float4 a4 = vals[p];
                 float v[4] = {a4.x + bias4[0], a4.y + bias4[1], a4.z + bias4[2], a4.w + bias4[3]};
@@ -436,7 +443,7 @@ __device__ __forceinline__ void gemm_tile(const Prob& pr, const int wg, char* sm
         // ... and all stores of the slab leave back to back
 #pragma unroll
         for (int p = 0; p < NP; p++) {
-            const int m = m_blk + wm * (BM / WM) + i * 32 + p * RPI + e_row;
+            const int m = m_blk + wm * (BM / WM) + i * SR + p * RPI + e_row;
             if (m < M && nvalid > 0) {
                 const long long idx = (long long)m * ldc + n0;
                 const float v[4] = {res[p].x, res[p].y, res[p].z, res[p].w};
@@ -515,6 +522,7 @@ template <int EPI, bool OUT_F32>
 int launch_epi(int variant, ProbSet& args, int n, hipStream_t st) {
     switch (variant) {
         case 4: return launch_cfg<256, 256, 2, 4, 2, EPI, OUT_F32>(args, n, st);
+        case 5: return launch_cfg<256, 192, 2, 4, 2, EPI, OUT_F32>(args, n, st);
         case 1: return launch_cfg<128, 128, 2, 2, 4, EPI, OUT_F32>(args, n, st);
         default: return launch_cfg<128, 128, 2, 2, 2, EPI, OUT_F32>(args, n, st);
     }
@@ -612,7 +620,8 @@ int gemm_bf16(const bf16_t* A, const bf16_t* Wp, void* out, int out_is_f32, int 
 }  // namespace sd3
 
 extern "C" int sd3_gemm_bf16_force_tile(int tile) {
-    if (tile != 0 && tile != 128 && tile != 256) return sd3::fail(SD3_ERR_INVALID_ARG, "sd3_gemm_bf16_force_tile: tile must be 0, 128 or 256 (got %d)", tile);
-    sd3::g_gemm_bf16_variant = tile == 0 ? -1 : (tile == 256 ? 4 : 0);
+    if (tile != 0 && tile != 128 && tile != 192 && tile != 256)
+        return sd3::fail(SD3_ERR_INVALID_ARG, "sd3_gemm_bf16_force_tile: tile must be 0, 128, 192 or 256 (got %d)", tile);
+    sd3::g_gemm_bf16_variant = tile == 0 ? -1 : (tile == 256 ? 4 : tile == 192 ? 5 : 0);
     return SD3_OK;
 }
