@@ -28,7 +28,13 @@ typedef enum sd3_status {
 
 typedef enum sd3_precision {
     SD3_PREC_F32 = 0, /* fp32 storage and fp32 MFMA arithmetic: matches the CPU reference to <= 1e-4 */
-    SD3_PREC_BF16 = 1 /* bf16 operands on the MFMA units, fp32 accumulation, fp32 residual stream */
+    SD3_PREC_BF16 = 1, /* bf16 operands on the MFMA units, fp32 accumulation, fp32 residual stream */
+    /* SD3_PREC_BF16 with the two MLP layers of both streams (half of the block's GEMM work) on the fp8 matrix instruction: OCP e4m3
+     * operands, fp32 accumulation; activations quantised per token row and weights per output channel ... */
+    SD3_PREC_BF16_FP8 = 2,
+    /* ... or with one factor per tensor on both sides (coarser; kept for comparison). Neither is the reference's arithmetic nor
+     * the benchmark's: they exist to be measured against the same error criterion as SD3_PREC_BF16. */
+    SD3_PREC_BF16_FP8_TENSOR = 3
 } sd3_precision;
 
 typedef enum sd3_activation { SD3_ACT_SILU = 0, SD3_ACT_GELU_TANH = 1 } sd3_activation;
@@ -160,7 +166,7 @@ int sd3_dit_forward_cfg_euler(sd3_ctx* ctx, const float* pooled, const float* ca
  * sd3_profile_end synchronises and returns, per class, the summed event time in ms, the summed algorithmic work
  * (FLOP for SD3_PROF_GEMM / SD3_PROF_ATTENTION: 2*M*N*K and 4*B*heads*Tq*Tk*head_dim; bytes for the others: each
  * tensor counted once per read and once per write) and the number of launches. Arrays have SD3_PROF_CLASSES entries. */
-enum { SD3_PROF_GEMM = 0, SD3_PROF_ATTENTION = 1, SD3_PROF_LAYERNORM = 2, SD3_PROF_ADALN = 3, SD3_PROF_CLASSES = 4 };
+enum { SD3_PROF_GEMM = 0, SD3_PROF_ATTENTION = 1, SD3_PROF_LAYERNORM = 2, SD3_PROF_ADALN = 3, SD3_PROF_GEMM_FP8 = 4, SD3_PROF_QUANT = 5, SD3_PROF_CLASSES = 6 };
 int sd3_profile_begin(sd3_ctx* ctx);
 int sd3_profile_end(sd3_ctx* ctx, double* ms, double* work, long long* launches);
 
@@ -204,6 +210,15 @@ typedef struct sd3_gemm_bf16_problem {
     const float* rms_k;
 } sd3_gemm_bf16_problem;
 int sd3_gemm_bf16_grouped(const sd3_gemm_bf16_problem* problems, int n_problems, int epilogue, int out_is_f32, void* stream);
+/* The fp8 form of the same GEMM (OCP e4m3 operands on v_mfma_f32_32x32x64_f8f6f4, fp32 accumulation), with no counterpart in the
+ * reference: out = epilogue(a_scale[m] * w_scale[n] * (Aq @ Wq^T) + bias).
+ * sd3_quantize_weight_fp8: W fp32 (K,N) in the reference's layout -> wq (N,K) bytes + w_scale (N): w_scale[n] = max_k |W[k][n]| / 448
+ * (per_tensor: the same factor, from the whole tensor, for every n). sd3_quantize_rows_fp8: A bf16 (M,K) -> aq (M,K) bytes +
+ * a_scale (M), one factor per row (per_tensor: one for all rows). K % 128 == 0. epilogue: 0 bias, 1 bias+GELU-tanh. */
+int sd3_quantize_weight_fp8(const float* W, void* wq, float* w_scale, int K, int N, int per_tensor, void* stream);
+int sd3_quantize_rows_fp8(const void* A, void* aq, float* a_scale, int M, int K, int per_tensor, void* stream);
+int sd3_gemm_fp8(const void* aq, const float* a_scale, const void* wq, const float* w_scale, const float* bias, void* out, int M, int N, int K, int epilogue,
+                 int out_is_f32, void* stream);
 /* fp32 -> bf16 (round to nearest even) */
 int sd3_cast_f32_to_bf16(const float* in, void* out, long long n, void* stream);
 /* Tuning hook with no counterpart in the reference: forces the output tile of the bf16 GEMM for every later call in this

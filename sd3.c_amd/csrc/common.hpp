@@ -100,6 +100,8 @@ struct GemmEpilogueArgs {
     const float* resid = nullptr;  // (M, ldc) fp32 for EPI_GATE_RESID
     const float* table = nullptr;  // (rows_per_batch, N) for EPI_BIAS_ROWADD
     int rows_per_batch = 1;
+    const float* a_scale = nullptr;  // fp8 GEMM: factor per row of A (M) and per output column (N); null = 1
+    const float* w_scale = nullptr;
 };
 
 // fp32 GEMM on the fp32 MFMA units: out(M,N) = A(M,K; lda) @ W(K, ldw)[:, n0:n0+N] (+ epilogue); out fp32 with row stride ldc.
@@ -118,6 +120,13 @@ struct GemmBf16Problem {
 };
 extern std::atomic<long long> g_gemm_bf16_launches;  // kernels launched by the bf16 GEMM so far (for per-launch profile figures)
 int gemm_bf16_grouped(const GemmBf16Problem* probs, int n, int out_is_f32, int epi, hipStream_t st);
+// The same with OCP fp8 (e4m3) operands: A (M,K) and Wp (N,K) are bytes, K % 128 == 0, and the accumulators are multiplied by
+// ea.a_scale[m] * ea.w_scale[n] before the epilogue (epilogues: bias, bias+GELU, gate+residual, q|k|v with qk-norm).
+int gemm_fp8_grouped(const GemmBf16Problem* probs, int n, int out_is_f32, int epi, hipStream_t st);
+// fp8 quantisation. Rows of a bf16 matrix: aq[m][k] = fp8(A[m][k] / s[m]), s[m] = max_k |A[m][k]| / 448 (one common s with per_tensor).
+int quantize_rows_fp8(const bf16_t* A, uint8_t* aq, float* scale, int M, int K, int per_tensor, hipStream_t st);
+// A (K,N) fp32 weight -> (N,K) fp8 with one factor per output column n (one common factor with per_tensor)
+int quantize_weight_fp8(const float* W, uint8_t* wq, float* scale, int K, int N, int per_tensor, hipStream_t st);
 // (K,N) fp32 row-major -> (N,K) bf16 row-major
 int pack_weight_bf16(const float* W, bf16_t* out, int K, int N, hipStream_t st);
 int cast_f32_to_bf16(const float* in, bf16_t* out, long long n, hipStream_t st);

@@ -58,8 +58,12 @@ static int static_scratch_of(int device, void** out) {
 struct PackedWeight {
     void* ptr = nullptr;
     long long K = 0, N = 0;
-    int kind = 0;  // 0: bf16 (N,K) transposed for the MFMA GEMM; 1: bf16 (K,N) plain cast for small_linear; 2: fp32 (K,N) transpose of an (N,K) tensor
+    int kind = 0;  // 0: bf16 (N,K) transposed for the MFMA GEMM; 1: bf16 (K,N) plain cast for small_linear; 2: fp32 (K,N) transpose of an (N,K) tensor;
+                   // 3 / 4: fp8 e4m3 (N,K) followed (at the next 256-byte boundary) by N fp32 factors, one per output column (3) or all equal (4)
 };
+static inline size_t fp8_scale_offset(long long K, long long N) { return ((size_t)K * N + 255) & ~(size_t)255; }
+static inline bool is_bf(int prec) { return prec != SD3_PREC_F32; }
+static inline int fp8_kind(int prec) { return prec == SD3_PREC_BF16_FP8 ? 3 : prec == SD3_PREC_BF16_FP8_TENSOR ? 4 : 0; }
 
 struct sd3_ctx {
     int device = 0;
@@ -147,7 +151,7 @@ int get_packed(sd3_ctx* ctx, const float* w, long long K, long long N, int kind,
     }
     PackedWeight p;
     p.K = K; p.N = N; p.kind = kind;
-    const size_t bytes = (size_t)K * N * (kind == 2 ? 4 : 2);
+    const size_t bytes = kind >= 3 ? fp8_scale_offset(K, N) + (size_t)N * sizeof(float) : (size_t)K * N * (kind == 2 ? 4 : 2);
     hipError_t e = hipMalloc(&p.ptr, bytes);
     if (e != hipSuccess) {
         (void)hipGetLastError();
@@ -156,6 +160,7 @@ int get_packed(sd3_ctx* ctx, const float* w, long long K, long long N, int kind,
     int rc;
     if (kind == 0) rc = pack_weight_bf16(w, (bf16_t*)p.ptr, (int)K, (int)N, ctx->stream);
     else if (kind == 1) rc = cast_f32_to_bf16(w, (bf16_t*)p.ptr, K * N, ctx->stream);
+    else if (kind >= 3) rc = quantize_weight_fp8(w, (uint8_t*)p.ptr, (float*)((char*)p.ptr + fp8_scale_offset(K, N)), (int)K, (int)N, kind == 4, ctx->stream);
     else rc = transpose_f32(w, (float*)p.ptr, (int)N, (int)K, ctx->stream);  // input is (N,K): transpose to (K,N)
     if (rc != SD3_OK) {
         (void)hipFree(p.ptr);
@@ -169,7 +174,7 @@ int get_packed(sd3_ctx* ctx, const float* w, long long K, long long N, int kind,
 // Frees every derived copy made from the tensor at `w` (after the work that may still read them has finished).
 int drop_packed_of(sd3_ctx* ctx, const float* w) {
     bool synced = false;
-    for (int kind = 0; kind < 3; kind++) {
+    for (int kind = 0; kind < 5; kind++) {
         auto it = ctx->packed.find(std::make_pair(w, kind));
         if (it == ctx->packed.end()) continue;
         if (!synced) {
@@ -226,9 +231,13 @@ struct Dims {
 
 size_t block_workspace_bytes(const Dims& d, int prec) {
     Bump b(nullptr, 0);
-    const size_t es = prec == SD3_PREC_BF16 ? 2 : 4;
+    const size_t es = is_bf(prec) ? 2 : 4;
     const size_t mc = (size_t)d.B * d.Tc, mx = (size_t)d.B * d.Tx;
     auto act = [&](size_t n) { b.take<char>(n * es); };
+    if (fp8_kind(prec)) {  // fp8 copies of the MLP inputs and one factor per row
+        b.take<char>(mc * d.E * d.C); b.take<char>(mx * d.E * d.C);
+        b.take<float>(mc); b.take<float>(mx);
+    }
     act(mc * d.C); act(mx * d.C); act(mx * d.C);           // c_hid, x_hid, x_hid2
     act(mc * 3 * d.C); act(mx * 3 * d.C);                  // c_qkv, x_qkv
     if (d.dual) act(mx * 3 * d.C);                         // x_qkv2
@@ -243,7 +252,7 @@ int linear_layer(sd3_ctx* ctx, int prec, const void* A, const float* W, const fl
                  GemmEpilogueArgs ea) {
     if (!W) return fail(SD3_ERR_MISSING_PARAM, "a weight needed by this configuration is not bound (N=%d K=%d)", N, K);
     ea.bias = bias;
-    if (prec == SD3_PREC_F32) {
+    if (!is_bf(prec)) {
         ProfScope ps(ctx, SD3_PROF_GEMM, 2.0 * M * N * K);
         return gemm_f32((const float*)A, K, W, N, 0, (float*)out, ldc, M, N, K, epi, ea, ctx->stream);
     }
@@ -264,7 +273,7 @@ struct LayerCall {
     GemmEpilogueArgs ea;
 };
 int linear_pair(sd3_ctx* ctx, int prec, const LayerCall* calls, int n, int out_f32, int epi) {
-    if (prec == SD3_PREC_F32) {
+    if (!is_bf(prec)) {
         for (int i = 0; i < n; i++) {
             const LayerCall& c = calls[i];
             if (c.M > 0) SD3_TRY(linear_layer(ctx, prec, c.A, c.W, c.bias, c.out, out_f32, c.ldc, c.M, c.N, c.K, epi, c.ea));
@@ -292,7 +301,7 @@ int linear_pair(sd3_ctx* ctx, int prec, const LayerCall* calls, int n, int out_f
 }
 
 int ada_jobs_run(sd3_ctx* ctx, int prec, const float* y, int B, int C, std::vector<SmallLinearJob>& jobs) {
-    if (prec == SD3_PREC_BF16) {
+    if (is_bf(prec)) {
         for (auto& j : jobs) {
             const void* wp = nullptr;
             SD3_TRY(get_packed(ctx, (const float*)j.W, C, j.ldw, 1, &wp));
@@ -300,9 +309,9 @@ int ada_jobs_run(sd3_ctx* ctx, int prec, const float* y, int B, int C, std::vect
         }
     }
     double bytes = 0;
-    for (auto& j : jobs) bytes += (double)C * j.N * (prec == SD3_PREC_BF16 ? 2 : 4) + (double)B * j.N * 4;
+    for (auto& j : jobs) bytes += (double)C * j.N * (is_bf(prec) ? 2 : 4) + (double)B * j.N * 4;
     ProfScope ps(ctx, SD3_PROF_ADALN, bytes, ((long long)jobs.size() + 15) / 16);  // one kernel per 16 weight matrices
-    return small_linear_batched(y, B, C, jobs.data(), (int)jobs.size(), prec == SD3_PREC_BF16, -1, ctx->stream);
+    return small_linear_batched(y, B, C, jobs.data(), (int)jobs.size(), is_bf(prec), -1, ctx->stream);
 }
 
 // LayerNorm + modulation, timed as a memory-bound launch: reads x once (fp32), writes one or two outputs.
@@ -338,9 +347,16 @@ int run_block(sd3_ctx* ctx, int prec, const float* y, float* c, float* x, const 
     const int B = d.B, Tc = d.Tc, Tx = d.Tx, C = d.C;
     const int mc = B * Tc, mx = B * Tx;
     const int cch = d.discard ? 2 : 6, xch = d.dual ? 9 : 6;
-    const bool bf = prec == SD3_PREC_BF16;
+    const bool bf = is_bf(prec);
+    const int f8 = fp8_kind(prec);
     const size_t es = bf ? 2 : 4;
     auto act = [&](size_t n) -> void* { return ws.take<char>(n * es); };
+    uint8_t *cq = nullptr, *xq = nullptr;
+    float *cs = nullptr, *xs = nullptr;
+    if (f8) {
+        cq = ws.take<uint8_t>((size_t)mc * d.E * C); xq = ws.take<uint8_t>((size_t)mx * d.E * C);
+        cs = ws.take<float>((size_t)mc); xs = ws.take<float>((size_t)mx);
+    }
     void* c_hid = act((size_t)mc * C);
     void* x_hid = act((size_t)mx * C);
     void* x_hid2 = act((size_t)mx * C);
@@ -453,6 +469,44 @@ int run_block(sd3_ctx* ctx, int prec, const float* y, float* c, float* x, const 
                                      {c, c_hid, nullptr, cchunk(3), cchunk(4), nullptr, nullptr, ldc_ada, B, d.discard ? 0 : Tc}};
         SD3_TRY(ln_mod_pair(ctx, ln2, 2, 1e-6f, C, bf));
     }
+    if (f8) {
+        // fp8 MLPs: the inputs of both layers are quantised row by row (one factor per token), the weights column by column (one
+        // factor per output channel) -- or one factor per tensor on either side -- and the products run on the fp8 matrix instruction
+        const int H = d.E * C;
+        auto fp8_pair = [&](const void* xa, const void* ca, int K, const float* xw, const float* cw, const float* xb, const float* cb, void* xo, void* co,
+                            int N, int out_f32, int epi, const GemmEpilogueArgs& xe, const GemmEpilogueArgs& ce) -> int {
+            {
+                ProfScope ps(ctx, SD3_PROF_QUANT, (double)(mx + mcm) * K * 3.0, mcm ? 4 : 2);
+                SD3_TRY(quantize_rows_fp8((const bf16_t*)xa, xq, xs, mx, K, f8 == 4, st));
+                SD3_TRY(quantize_rows_fp8((const bf16_t*)ca, cq, cs, mcm, K, f8 == 4, st));
+            }
+            GemmBf16Problem probs[2];
+            int n = 0;
+            double flop = 0;
+            const void* wp = nullptr;
+            if (!xw) return fail(SD3_ERR_MISSING_PARAM, "a weight needed by this configuration is not bound (N=%d K=%d)", N, K);
+            SD3_TRY(get_packed(ctx, xw, K, N, f8, &wp));
+            probs[n] = GemmBf16Problem{(const bf16_t*)xq, (const bf16_t*)wp, xo, N, mx, N, K, xe};
+            probs[n].ea.bias = xb; probs[n].ea.a_scale = xs; probs[n].ea.w_scale = (const float*)((const char*)wp + fp8_scale_offset(K, N));
+            flop += 2.0 * mx * N * K;
+            n++;
+            if (mcm > 0) {
+                if (!cw) return fail(SD3_ERR_MISSING_PARAM, "a weight needed by this configuration is not bound (N=%d K=%d)", N, K);
+                SD3_TRY(get_packed(ctx, cw, K, N, f8, &wp));
+                probs[n] = GemmBf16Problem{(const bf16_t*)cq, (const bf16_t*)wp, co, N, mcm, N, K, ce};
+                probs[n].ea.bias = cb; probs[n].ea.a_scale = cs; probs[n].ea.w_scale = (const float*)((const char*)wp + fp8_scale_offset(K, N));
+                flop += 2.0 * mcm * N * K;
+                n++;
+            }
+            ProfScope ps(ctx, SD3_PROF_GEMM_FP8, flop);
+            return gemm_fp8_grouped(probs, n, out_f32, epi, st);
+        };
+        SD3_TRY(fp8_pair(x_hid, c_hid, C, w.x_mlp_w1, w.c_mlp_w1, w.x_mlp_b1, w.c_mlp_b1, x_mlp, c_mlp, H, 0, EPI_BIAS_GELU, none, none));
+        gc.gate = cchunk(5);
+        gx.gate = xchunk(5);
+        SD3_TRY(fp8_pair(x_mlp, c_mlp, H, w.x_mlp_w2, w.c_mlp_w2, w.x_mlp_b2, w.c_mlp_b2, x, c, C, 1, EPI_GATE_RESID, gx, gc));
+        return SD3_OK;
+    }
     {
         LayerCall up[2] = {{x_hid, w.x_mlp_w1, w.x_mlp_b1, x_mlp, d.E * C, mx, d.E * C, C, none},
                            {c_hid, w.c_mlp_w1, w.c_mlp_b1, c_mlp, d.E * C, mcm, d.E * C, C, none}};
@@ -470,8 +524,9 @@ int check_block_dims(const Dims& d, int prec) {
         return fail(SD3_ERR_INVALID_ARG, "block: sizes must be positive (B=%d Tc=%d Tx=%d emb_dim=%d heads=%d mlp_expand=%d)", d.B, d.Tc, d.Tx, d.C, d.NH, d.E);
     if (d.C % d.NH) return fail(SD3_ERR_INVALID_ARG, "block: emb_dim %d is not divisible by attn_heads %d", d.C, d.NH);
     if (d.B > 8) return fail(SD3_ERR_UNSUPPORTED, "block: batch %d > 8", d.B);
-    if (prec != SD3_PREC_F32 && prec != SD3_PREC_BF16) return fail(SD3_ERR_INVALID_ARG, "unknown precision %d", prec);
-    if (prec == SD3_PREC_BF16 && (d.HS != 64 || d.C % 64)) return fail(SD3_ERR_UNSUPPORTED, "bf16 path needs head_dim 64 and emb_dim %% 64 == 0");
+    if (prec < SD3_PREC_F32 || prec > SD3_PREC_BF16_FP8_TENSOR) return fail(SD3_ERR_INVALID_ARG, "unknown precision %d", prec);
+    if (is_bf(prec) && (d.HS != 64 || d.C % 64)) return fail(SD3_ERR_UNSUPPORTED, "bf16 path needs head_dim 64 and emb_dim %% 64 == 0");
+    if (fp8_kind(prec) && (d.C % 128)) return fail(SD3_ERR_UNSUPPORTED, "fp8 MLPs need emb_dim %% 128 == 0");
     if (prec == SD3_PREC_F32 && d.HS > 128) return fail(SD3_ERR_UNSUPPORTED, "fp32 path needs head_dim <= 128");
     return SD3_OK;
 }
@@ -754,7 +809,7 @@ int sd3_weights_bind(sd3_ctx* ctx, const char* name, const float* ptr, long long
 }
 int sd3_weights_prepare(sd3_ctx* ctx, int precision) {
     NOTNULL(ctx);
-    SD3_REQUIRE(precision == SD3_PREC_F32 || precision == SD3_PREC_BF16, "weights_prepare: unknown precision %d", precision);
+    SD3_REQUIRE(precision >= SD3_PREC_F32 && precision <= SD3_PREC_BF16_FP8_TENSOR, "weights_prepare: unknown precision %d", precision);
     DeviceGuard g(ctx->device);
     if (!g.ok) return fail(SD3_ERR_HIP, "cannot select device %d", ctx->device);
     // drop what exists (the bound tensors may have been changed in place) ...
@@ -775,11 +830,15 @@ int sd3_weights_prepare(sd3_ctx* ctx, int precision) {
         const long long N = b->second.second, K = kv.second.second / N;
         const void* unused = nullptr;
         if (name == "to_patch.conv.weight") {  // (C_out, C_in*p*p): bf16 cast for the MFMA GEMM, fp32 transpose for the fp32 one
-            if (precision == SD3_PREC_BF16) SD3_TRY(get_packed(ctx, kv.second.first, N, K, 1, &unused));
+            if (is_bf(precision)) SD3_TRY(get_packed(ctx, kv.second.first, N, K, 1, &unused));
             else SD3_TRY(get_packed(ctx, kv.second.first, K, N, 2, &unused));
             continue;
         }
-        if (precision != SD3_PREC_BF16) continue;
+        if (!is_bf(precision)) continue;
+        if (fp8_kind(precision) && (ends_with(name, "_mlp.lin1.weight") || ends_with(name, "_mlp.lin2.weight")) && K % 128 == 0) {
+            SD3_TRY(get_packed(ctx, kv.second.first, K, N, fp8_kind(precision), &unused));
+            continue;
+        }
         const bool adaln = ends_with(name, "ada_lnorm.linear.weight") || name == "ada_ln_out.linear.weight";
         const bool gemm = ends_with(name, "_to_qkv.weight") || ends_with(name, "_attn_Wout.weight") || ends_with(name, "_mlp.lin1.weight") ||
                           ends_with(name, "_mlp.lin2.weight") || name == "captions_linear.weight" || name == "linear_out.weight";
@@ -894,7 +953,7 @@ static int dit_forward_impl(sd3_ctx* ctx, const float* pooled, const float* capt
     SD3_REQUIRE(C % 4 == 0, "DiT: emb_dim must be a multiple of 4");
     Dims dmax{B, Tc, Tx, C, attn_heads, C / attn_heads, mlp_expand, n_dual > 0, use_qk_norm != 0, false};
     SD3_TRY(check_block_dims(dmax, precision));
-    const bool bf = precision == SD3_PREC_BF16;
+    const bool bf = is_bf(precision);
     if (bf && ((captions_dim % 64) || (Kp % 64))) return fail(SD3_ERR_UNSUPPORTED, "bf16 path needs captions_dim and C_in*patch^2 to be multiples of 64");
     DeviceGuard g(ctx->device);
     if (!g.ok) return fail(SD3_ERR_HIP, "cannot select device %d", ctx->device);
@@ -1128,6 +1187,27 @@ int sd3_gemm_bf16_grouped(const sd3_gemm_bf16_problem* problems, int n_problems,
         probs[i] = GemmBf16Problem{(const bf16_t*)q.A, (const bf16_t*)q.wpacked, q.out, q.N, q.M, q.N, q.K, ea};
     }
     return gemm_bf16_grouped(probs, n_problems, out_is_f32, epilogue, ST(stream));
+}
+int sd3_quantize_weight_fp8(const float* W, void* wq, float* w_scale, int K, int N, int per_tensor, void* stream) {
+    SD3_REQUIRE(K > 0 && N > 0, "quantize_weight_fp8: bad sizes");
+    NOTNULL(W); NOTNULL(wq); NOTNULL(w_scale);
+    return quantize_weight_fp8(W, (uint8_t*)wq, w_scale, K, N, per_tensor != 0, ST(stream));
+}
+int sd3_quantize_rows_fp8(const void* A, void* aq, float* a_scale, int M, int K, int per_tensor, void* stream) {
+    SD3_REQUIRE(M >= 0 && K > 0, "quantize_rows_fp8: bad sizes");
+    if (M == 0) return SD3_OK;
+    NOTNULL(A); NOTNULL(aq); NOTNULL(a_scale);
+    return quantize_rows_fp8((const bf16_t*)A, (uint8_t*)aq, a_scale, M, K, per_tensor != 0, ST(stream));
+}
+int sd3_gemm_fp8(const void* aq, const float* a_scale, const void* wq, const float* w_scale, const float* bias, void* out, int M, int N, int K, int epilogue,
+                 int out_is_f32, void* stream) {
+    SD3_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_fp8: bad sizes");
+    SD3_REQUIRE(epilogue == EPI_BIAS || epilogue == EPI_BIAS_GELU, "gemm_fp8: epilogue must be 0 (bias) or 1 (bias+GELU)");
+    if (M == 0) return SD3_OK;
+    NOTNULL(aq); NOTNULL(wq); NOTNULL(out);
+    GemmBf16Problem q{(const bf16_t*)aq, (const bf16_t*)wq, out, N, M, N, K, GemmEpilogueArgs{}};
+    q.ea.bias = bias; q.ea.a_scale = a_scale; q.ea.w_scale = w_scale;
+    return gemm_fp8_grouped(&q, 1, out_is_f32, epilogue, ST(stream));
 }
 int sd3_cast_f32_to_bf16(const float* in, void* out, long long n, void* stream) {
     SD3_REQUIRE(n >= 0, "cast: negative size");

@@ -20,6 +20,8 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 typedef const __attribute__((address_space(1))) void* glb_ptr_t;
 
 struct EpiDev {
+    const float* a_scale;  // fp8 operands: one factor per row of A (null: 1)
+    const float* w_scale;  // fp8 operands: one factor per output column (null: 1)
     const float* bias;
     const float* gate;
     const float* resid;
@@ -78,10 +80,16 @@ struct ProbSet {
 };
 
 // One output tile: K loop + epilogue. `wg` is the tile's position in the XCD-aware order of its problem.
-template <int BM, int BN, int WM, int WN, int STAGES, int EPI, bool OUT_F32>
+typedef __attribute__((__vector_size__(8 * sizeof(int)))) int i32x8_t;
+typedef __attribute__((__vector_size__(4 * sizeof(int)))) int i32x4_t;
+
+// FP8: the operands are OCP e4m3 bytes (A (M,K) and Wp (N,K), both K-contiguous); a 128-byte LDS row then holds 128 k values and
+// the matrix instruction is v_mfma_f32_32x32x64_f8f6f4; the accumulators are multiplied by a_scale[m] * w_scale[n] in the epilogue.
+template <int BM, int BN, int WM, int WN, int STAGES, int EPI, bool OUT_F32, bool FP8>
 __device__ __forceinline__ void gemm_tile(const Prob& pr, const int wg, char* smem) {
-    const bf16_t* __restrict__ A = pr.A;
-    const bf16_t* __restrict__ Wp = pr.Wp;
+    constexpr int ESZ = FP8 ? 1 : 2;                  // bytes per operand element
+    const char* __restrict__ A = reinterpret_cast<const char*>(pr.A);
+    const char* __restrict__ Wp = reinterpret_cast<const char*>(pr.Wp);
     void* __restrict__ out_ = pr.out;
     const int ldc = pr.ldc, M = pr.M, N = pr.N, K = pr.K;
     const EpiDev epi = pr.epi;
@@ -100,34 +108,35 @@ __device__ __forceinline__ void gemm_tile(const Prob& pr, const int wg, char* sm
     const int m_blk = tile_m * BM, n_blk = tile_n * BN;
 
     // ---- loader: chunk q = i*NT + tid lands at LDS byte q*16 of its tile, i.e. row q/8, physical chunk q%8 ----
-    const bf16_t* ga[LA];
-    const bf16_t* gb[LB];
+    const char* ga[LA];
+    const char* gb[LB];
+    const long long row_bytes = (long long)K * ESZ;
 #pragma unroll
     for (int i = 0; i < LA; i++) {
         const int q = i * NT + tid, row = q >> 3, lc = (q & 7) ^ swz(row);
         const int m = min(m_blk + row, M - 1);  // rows beyond M re-read the last row; their results are never stored
-        ga[i] = A + (long long)m * K + lc * 8;
+        ga[i] = A + (long long)m * row_bytes + lc * 16;
     }
 #pragma unroll
     for (int i = 0; i < LB; i++) {
         const int q = i * NT + tid, row = q >> 3, lc = (q & 7) ^ swz(row);
         const int n = min(n_blk + row, N - 1);
-        gb[i] = Wp + (long long)n * K + lc * 8;
+        gb[i] = Wp + (long long)n * row_bytes + lc * 16;
     }
     auto issue_tile = [&](int kt, int stage) {
         char* sa = smem + stage * STAGE_BYTES + wave * 1024;
         char* sb = sa + A_BYTES;
 #pragma unroll
-        for (int i = 0; i < LA; i++) __builtin_amdgcn_global_load_lds((glb_ptr_t)(ga[i] + kt * BK), (lds_ptr_t)(sa + i * NT * 16), 16, 0, 0);
+        for (int i = 0; i < LA; i++) __builtin_amdgcn_global_load_lds((glb_ptr_t)(ga[i] + kt * 128), (lds_ptr_t)(sa + i * NT * 16), 16, 0, 0);
 #pragma unroll
-        for (int i = 0; i < LB; i++) __builtin_amdgcn_global_load_lds((glb_ptr_t)(gb[i] + kt * BK), (lds_ptr_t)(sb + i * NT * 16), 16, 0, 0);
+        for (int i = 0; i < LB; i++) __builtin_amdgcn_global_load_lds((glb_ptr_t)(gb[i] + kt * 128), (lds_ptr_t)(sb + i * NT * 16), 16, 0, 0);
     };
 
     // Two matrix instructions. 256x256 tiles use v_mfma_f32_16x16x32_bf16: on this device the clock under matrix load is set by
     // the power limit, and measured on random operands the 16x16x32 form sustains 15-24 % more than 32x32x16 at the same nominal
     // rate (half as many accumulator updates per product). 128x128 tiles keep v_mfma_f32_32x32x16_bf16: with four wavefronts per
     // workgroup the finer instruction stream measured 5-15 % slower there. Both forms give bit-identical results.
-    constexpr bool M16 = (BM == 256);
+    constexpr bool M16 = (BM == 256) && !FP8;
     constexpr int MI = BM / WM / 16, NJ = BN / WN / 16;      // 16x16 blocks per wavefront
     f32x16_t acc[M16 ? 1 : TM][M16 ? 1 : TN];
     f32x4_t acc16[M16 ? MI : 1][M16 ? NJ : 1];
@@ -145,7 +154,7 @@ __device__ __forceinline__ void gemm_tile(const Prob& pr, const int wg, char* sm
             for (int r = 0; r < 4; r++) acc16[i][j][r] = 0.f;
 
     static_assert(STAGES >= 2 && (STAGES - 1) * (LA + LB) < 64, "ring depth: at least two stages, and the loads in flight must fit the 6-bit counter");
-    const int nkt = K / BK;
+    const int nkt = (int)(row_bytes / 128);
     const int l32 = lane & 31, lk = lane >> 5;   // position in a 32x32 block
     const int lr = lane & 15, lg = lane >> 4;    // position in a 16x16 block
 
@@ -233,18 +242,29 @@ __device__ __forceinline__ void gemm_tile(const Prob& pr, const int wg, char* sm
         for (int kt = 0; kt + 1 < nkt; kt++) k_tile(kt, std::true_type{});
         k_tile(nkt - 1, std::false_type{});
     } else {
-        // operand addresses inside a stage: row*128 + ((2*ks + lk) ^ sw)*16 with sw = swz(row) = swz(l32) (block offsets are multiples of 16)
+        // operand addresses inside a stage: row*128 + (chunk ^ sw)*16 with sw = swz(row) = swz(l32) (block offsets are multiples of 16).
+        // bf16: k-step ks (16 deep) takes chunk 2*ks + lk; fp8: k-step ks (64 deep) takes the two chunks 4*ks + 2*lk, +1
         const int sw = swz(l32);
         const int a_off = (wm * (BM / WM) + l32) * 128, b_off = A_BYTES + (wn * (BN / WN) + l32) * 128;
         // operand fragments of k-step ks live in buffer ks&1; those of step ks+1 are fetched from LDS while the matrix cores work on step ks
-        bf16x8_t a[2][TM], b[2][TN];
-        auto fetch = [&](const char* st, int ks, int buf) {
-            const int ch = ((2 * ks + lk) ^ sw) * 16;
-#pragma unroll
-            for (int i = 0; i < TM; i++) a[buf][i] = *reinterpret_cast<const bf16x8_t*>(st + a_off + i * 32 * 128 + ch);
-#pragma unroll
-            for (int j = 0; j < TN; j++) b[buf][j] = *reinterpret_cast<const bf16x8_t*>(st + b_off + j * 32 * 128 + ch);
+        using frag_t = std::conditional_t<FP8, i32x8_t, bf16x8_t>;
+        frag_t a[2][TM], b[2][TN];
+        auto read_frag = [&](const char* row, int ks) -> frag_t {
+            if constexpr (FP8) {
+                const i32x4_t lo = *reinterpret_cast<const i32x4_t*>(row + (((4 * ks + 2 * lk) ^ sw) * 16));
+                const i32x4_t hi = *reinterpret_cast<const i32x4_t*>(row + (((4 * ks + 2 * lk + 1) ^ sw) * 16));
+                return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+            } else {
+                return *reinterpret_cast<const bf16x8_t*>(row + (((2 * ks + lk) ^ sw) * 16));
+            }
         };
+        auto fetch = [&](const char* st, int ks, int buf) {
+#pragma unroll
+            for (int i = 0; i < TM; i++) a[buf][i] = read_frag(st + a_off + i * 32 * 128, ks);
+#pragma unroll
+            for (int j = 0; j < TN; j++) b[buf][j] = read_frag(st + b_off + j * 32 * 128, ks);
+        };
+        constexpr int DSR = FP8 ? 2 : 1;  // LDS reads per fragment
 
         // Every stage is filled up front and exactly one tile is requested per K tile after that (past the end: the last tile
         // once more, into a buffer nobody reads again), so "tile kt+1 has landed" is always "all but the newest STAGES-2 tiles".
@@ -256,9 +276,9 @@ __device__ __forceinline__ void gemm_tile(const Prob& pr, const int wg, char* sm
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
         fetch(smem, 0, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, TM + TN, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, DSR * (TM + TN), 0);
 
-        constexpr int KS = BK / 16;
+        constexpr int KS = FP8 ? 2 : 4;  // k-steps per 128-byte K tile
         // One K tile. The workgroup barrier sits in front of the LAST k-step of a tile, not behind it: by then every fragment
         // of tile kt is in registers (or on its way: waited for), so its buffer can be handed to the loads of tile kt+2, and the
         // loads' issue and the first fragment reads of tile kt+1 are interleaved with the matrix instructions of that last
@@ -271,7 +291,10 @@ __device__ __forceinline__ void gemm_tile(const Prob& pr, const int wg, char* sm
 #pragma unroll
                 for (int i = 0; i < TM; i++)
 #pragma unroll
-                    for (int j = 0; j < TN; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[buf][i], b[buf][j], acc[i][j], 0, 0, 0);
+                    for (int j = 0; j < TN; j++) {
+                        if constexpr (FP8) acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a[buf][i], b[buf][j], acc[i][j], 0, 0, 0, 0, 0, 0);
+                        else acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[buf][i], b[buf][j], acc[i][j], 0, 0, 0);
+                    }
             };
             // scheduling pattern of a step: behind each of the first matrix instructions one LDS fragment read of the next step
             // (and, in the last step, one direct global->LDS load of the tile after next), so that their issue and latency are
@@ -282,8 +305,8 @@ __device__ __forceinline__ void gemm_tile(const Prob& pr, const int wg, char* sm
                 mfmas(ks & 1);
 #pragma unroll
                 for (int x = 0; x < TM + TN; x++) {
-                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
-                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // 1 DS read
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);    // 1 MFMA
+                    __builtin_amdgcn_sched_group_barrier(0x100, DSR, 0);  // 1 fragment read
                 }
                 __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - (TM + TN), 0);
             }
@@ -305,7 +328,7 @@ __device__ __forceinline__ void gemm_tile(const Prob& pr, const int wg, char* sm
 #pragma unroll
                 for (int x = 0; x < NM; x++) {
                     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                              // 1 MFMA
-                    if (x < TM + TN) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);              // 1 DS read
+                    if (x < TM + TN) __builtin_amdgcn_sched_group_barrier(0x100, DSR, 0);            // 1 fragment read
                     if (x * LPS < NLOADS) __builtin_amdgcn_sched_group_barrier(0x020, LPS, 0);       // VMEM reads
                 }
             }
@@ -343,6 +366,11 @@ __device__ __forceinline__ void gemm_tile(const Prob& pr, const int wg, char* sm
 #pragma unroll
         for (int c = 0; c < 4; c++)
             if (c < nvalid) bias4[c] = epi.bias[n0 + c];
+    float ws4[4] = {1.f, 1.f, 1.f, 1.f};  // fp8: the output column's factor
+    if (FP8 && epi.w_scale)
+#pragma unroll
+        for (int c = 0; c < 4; c++)
+            if (c < nvalid) ws4[c] = epi.w_scale[n0 + c];
     // batch index of a row without a division per row: the tile starts in batch b0 and crosses a boundary every rpb rows
     const int rpb = epi.rows_per_batch, b0 = m_blk / rpb;
     // gated layers: the residual rows of the NEXT slab are requested before the current slab goes through LDS, so that
@@ -394,7 +422,11 @@ __device__ __forceinline__ void gemm_tile(const Prob& pr, const int wg, char* sm
             const int row = p * RPI + e_row;
             const int m = m_blk + wm * (BM / WM) + i * SR + row;
             if (m < M && nvalid > 0) {
-                const float4 a4 = vals[p];
+                float4 a4 = vals[p];
+                if constexpr (FP8) {
+                    const float sa = epi.a_scale ? epi.a_scale[m] : 1.0f;
+                    a4.x *= sa * ws4[0]; a4.y *= sa * ws4[1]; a4.z *= sa * ws4[2]; a4.w *= sa * ws4[3];
+                }
                 float v[4] = {a4.x + bias4[0], a4.y + bias4[1], a4.z + bias4[2], a4.w + bias4[3]};
                 const long long idx = (long long)m * ldc + n0;
                 if (EPI == EPI_BIAS_GELU) {
@@ -467,12 +499,12 @@ __device__ __forceinline__ void gemm_tile(const Prob& pr, const int wg, char* sm
 // Persistent kernel: one workgroup per compute unit walks over the tiles of up to three problems. The stores of a finished
 // tile drain while the next tile's K loop is already running, instead of holding the compute unit until they retire.
 // Workgroup g takes work items g, g + G, g + 2G ... (G = grid size, a multiple of 8), so it stays on its XCD's run of tiles.
-template <int BM, int BN, int WM, int WN, int STAGES, int EPI, bool OUT_F32>
+template <int BM, int BN, int WM, int WN, int STAGES, int EPI, bool OUT_F32, bool FP8 = false>
 __global__ void __launch_bounds__(WM* WN * 64) gemm_bf16_kernel(const ProbSet args) {
     extern __shared__ __attribute__((aligned(1024))) char smem[];
     for (int w = blockIdx.x; w < args.end[MAX_PROBS - 1]; w += gridDim.x) {
         const int which = (w >= args.end[0]) + (w >= args.end[1]);
-        gemm_tile<BM, BN, WM, WN, STAGES, EPI, OUT_F32>(args.p[which], w - (which ? args.end[which - 1] : 0), smem);
+        gemm_tile<BM, BN, WM, WN, STAGES, EPI, OUT_F32, FP8>(args.p[which], w - (which ? args.end[which - 1] : 0), smem);
         __syncthreads();  // the staging slabs of this tile's epilogue alias the ring the next tile fills
     }
 }
@@ -491,9 +523,9 @@ int compute_units() {
     return cus;
 }
 
-template <int BM, int BN, int WM, int WN, int STAGES, int EPI, bool OUT_F32>
+template <int BM, int BN, int WM, int WN, int STAGES, int EPI, bool OUT_F32, bool FP8 = false>
 int launch_cfg(ProbSet& args, int n, hipStream_t st) {
-    auto kern = gemm_bf16_kernel<BM, BN, WM, WN, STAGES, EPI, OUT_F32>;
+    auto kern = gemm_bf16_kernel<BM, BN, WM, WN, STAGES, EPI, OUT_F32, FP8>;
     constexpr int smem = smem_bytes<BM, BN, WM, WN, STAGES>();
     static bool attr_done = false;  // raising the dynamic LDS limit is a per-function, per-process setting
     if (smem > 65536 && !attr_done) {
@@ -518,6 +550,13 @@ int launch_cfg(ProbSet& args, int n, hipStream_t st) {
     return launch_status("gemm_bf16");
 }
 
+// fp8 operands: 256x256 tiles (variant 4) or 128x128 tiles with a ring of two stages (anything else)
+template <int EPI, bool OUT_F32>
+int launch_epi_fp8(int variant, ProbSet& args, int n, hipStream_t st) {
+    if (variant == 4) return launch_cfg<256, 256, 2, 4, 2, EPI, OUT_F32, true>(args, n, st);
+    return launch_cfg<128, 128, 2, 2, 2, EPI, OUT_F32, true>(args, n, st);
+}
+
 template <int EPI, bool OUT_F32>
 int launch_epi(int variant, ProbSet& args, int n, hipStream_t st) {
     switch (variant) {
@@ -533,19 +572,21 @@ int launch_epi(int variant, ProbSet& args, int n, hipStream_t st) {
 std::atomic<long long> g_gemm_bf16_launches{0};
 int g_gemm_bf16_variant = -1;  // -1: choose by shape; 0 / 4: forced 128x128 / 256x256 tiles (sd3_gemm_bf16_force_tile); 1: 128x128 with a ring of four stages
 
-int gemm_bf16_grouped(const GemmBf16Problem* probs, int n, int out_is_f32, int epi, hipStream_t st) {
+static int grouped_impl(const GemmBf16Problem* probs, int n, int out_is_f32, int epi, bool fp8, hipStream_t st) {
     if (n < 1 || n > MAX_PROBS) return fail(SD3_ERR_INVALID_ARG, "gemm_bf16_grouped: 1 to %d problems (got %d)", MAX_PROBS, n);
     ProbSet args{};
     int m = 0, max_M = 0;
     for (int i = 0; i < n; i++) {
         const GemmBf16Problem& q = probs[i];
         if (q.M <= 0 || q.N <= 0) continue;  // an empty problem simply contributes no tiles
-        if (q.K <= 0 || (q.K % BK) != 0) return fail(SD3_ERR_UNSUPPORTED, "gemm_bf16: K=%d must be a positive multiple of %d", q.K, BK);
+        const int kmult = fp8 ? 128 : BK;  // one LDS row of a K tile is 128 bytes
+        if (q.K <= 0 || (q.K % kmult) != 0) return fail(SD3_ERR_UNSUPPORTED, "gemm_%s: K=%d must be a positive multiple of %d", fp8 ? "fp8" : "bf16", q.K, kmult);
         if ((reinterpret_cast<uintptr_t>(q.A) & 15) || (reinterpret_cast<uintptr_t>(q.Wp) & 15))
             return fail(SD3_ERR_INVALID_ARG, "gemm_bf16: operands must be 16-byte aligned");
         Prob& d = args.p[m++];
         d.A = q.A; d.Wp = q.Wp; d.out = q.out; d.ldc = q.ldc; d.M = q.M; d.N = q.N; d.K = q.K;
-        d.epi = EpiDev{q.ea.bias, q.ea.gate, q.ea.resid, q.ea.table, q.ea.gate_ld, q.ea.rows_per_batch > 0 ? q.ea.rows_per_batch : 1};
+        d.epi = EpiDev{fp8 ? q.ea.a_scale : nullptr, fp8 ? q.ea.w_scale : nullptr, q.ea.bias, q.ea.gate, q.ea.resid, q.ea.table, q.ea.gate_ld,
+                       q.ea.rows_per_batch > 0 ? q.ea.rows_per_batch : 1};
         if (epi == EPI_BIAS_ROWADD) d.epi.gate_ld = q.N;
         if (epi == EPI_QKV_NORM) {
             if (q.N % 192 || !q.ea.gate || !q.ea.resid || (reinterpret_cast<uintptr_t>(q.ea.gate) & 15) || (reinterpret_cast<uintptr_t>(q.ea.resid) & 15))
@@ -556,6 +597,17 @@ int gemm_bf16_grouped(const GemmBf16Problem* probs, int n, int out_is_f32, int e
     }
     if (m == 0) return SD3_OK;
     auto launch = [&](ProbSet& pp, int count, int v) -> int {
+        if (fp8) {
+#define SD3_GEMM_FP8_LAUNCH(E) return out_is_f32 ? launch_epi_fp8<E, true>(v, pp, count, st) : launch_epi_fp8<E, false>(v, pp, count, st)
+            switch (epi) {
+                case EPI_BIAS: SD3_GEMM_FP8_LAUNCH(EPI_BIAS);
+                case EPI_BIAS_GELU: SD3_GEMM_FP8_LAUNCH(EPI_BIAS_GELU);
+                case EPI_GATE_RESID: SD3_GEMM_FP8_LAUNCH(EPI_GATE_RESID);
+                case EPI_QKV_NORM: SD3_GEMM_FP8_LAUNCH(EPI_QKV_NORM);
+                default: return fail(SD3_ERR_UNSUPPORTED, "gemm_fp8: epilogue %d is not built for fp8 operands", epi);
+            }
+#undef SD3_GEMM_FP8_LAUNCH
+        }
 #define SD3_GEMM_BF16_LAUNCH(E) return out_is_f32 ? launch_epi<E, true>(v, pp, count, st) : launch_epi<E, false>(v, pp, count, st)
         switch (epi) {
             case EPI_BIAS: SD3_GEMM_BF16_LAUNCH(EPI_BIAS);
@@ -568,7 +620,7 @@ int gemm_bf16_grouped(const GemmBf16Problem* probs, int n, int out_is_f32, int e
         }
 #undef SD3_GEMM_BF16_LAUNCH
     };
-    if (g_gemm_bf16_variant >= 0) return launch(args, m, g_gemm_bf16_variant);
+    if (g_gemm_bf16_variant >= 0) return launch(args, m, fp8 && g_gemm_bf16_variant != 4 ? 0 : g_gemm_bf16_variant);
     // Tile shape and grouping by a small cost model. A persistent launch takes ceil(tiles / resident workgroups) rounds; the unit
     // of cost is one round of 256x256 tiles (8 wavefronts, one workgroup per compute unit). Measured on full rounds, a round of
     // 128x128 tiles (4 wavefronts, two workgroups per unit) takes 0.62 of that for a quarter of the outputs per tile, and a launch
@@ -610,6 +662,9 @@ int gemm_bf16_grouped(const GemmBf16Problem* probs, int n, int out_is_f32, int e
     }
     return launch(args, m, plan == 0 ? 4 : 0);
 }
+
+int gemm_bf16_grouped(const GemmBf16Problem* probs, int n, int out_is_f32, int epi, hipStream_t st) { return grouped_impl(probs, n, out_is_f32, epi, false, st); }
+int gemm_fp8_grouped(const GemmBf16Problem* probs, int n, int out_is_f32, int epi, hipStream_t st) { return grouped_impl(probs, n, out_is_f32, epi, true, st); }
 
 int gemm_bf16(const bf16_t* A, const bf16_t* Wp, void* out, int out_is_f32, int ldc, int M, int N, int K, int epi, const GemmEpilogueArgs& ea,
               hipStream_t st) {

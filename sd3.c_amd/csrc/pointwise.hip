@@ -560,3 +560,112 @@ int unpatchify_cfg_euler(const float* tokens, const float* latent, float* out, i
 }
 
 }  // namespace sd3
+
+// ---- OCP fp8 (e4m3) quantisation for the fp8 GEMM ----
+namespace sd3 {
+namespace {
+constexpr float FP8_MAX = 448.0f;  // largest finite e4m3 value
+
+__device__ __forceinline__ uint32_t pack_fp8x4(float a, float b, float c, float d) {
+    int v = 0;
+    v = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, v, false);
+    v = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, v, true);
+    return (uint32_t)v;
+}
+
+// one wavefront per row: amax[m] = max_k |A[m][k]|
+__global__ void __launch_bounds__(256) row_amax_bf16_kernel(const bf16_t* __restrict__ A, float* __restrict__ amax, int M, int K) {
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    if (row >= M) return;
+    const uint2* p = reinterpret_cast<const uint2*>(A + (long long)row * K);  // 4 bf16 per load (K % 4 == 0)
+    float mx = 0.f;
+    for (int i = lane; i < K / 4; i += 64) {
+        const uint2 v = p[i];
+        mx = fmaxf(mx, fmaxf(fmaxf(fabsf(__uint_as_float(v.x << 16)), fabsf(__uint_as_float(v.x & 0xffff0000u))),
+                             fmaxf(fabsf(__uint_as_float(v.y << 16)), fabsf(__uint_as_float(v.y & 0xffff0000u)))));
+    }
+    mx = wave_max(mx);
+    if (lane == 0) amax[row] = mx;
+}
+// vals[i] <- max over all i (one workgroup; fixed order, so the result does not depend on timing)
+__global__ void __launch_bounds__(1024) broadcast_max_kernel(float* __restrict__ vals, int n) {
+    __shared__ float part[16];
+    float mx = 0.f;
+    for (int i = threadIdx.x; i < n; i += 1024) mx = fmaxf(mx, vals[i]);
+    mx = wave_max(mx);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = mx;
+    __syncthreads();
+    mx = 0.f;
+    for (int i = 0; i < 16; i++) mx = fmaxf(mx, part[i]);
+    __syncthreads();
+    for (int i = threadIdx.x; i < n; i += 1024) vals[i] = mx;
+}
+// aq[m][k] = fp8(A[m][k] / s), s = amax[m] / 448 (1 for an all-zero row); amax[m] is overwritten with s
+__global__ void __launch_bounds__(256) quantize_rows_fp8_kernel(const bf16_t* __restrict__ A, uint8_t* __restrict__ aq, float* __restrict__ amax, int M, int K) {
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    if (row >= M) return;
+    const float mx = amax[row];
+    const float s = mx > 0.f ? mx * (1.0f / FP8_MAX) : 1.0f, inv = 1.0f / s;
+    const uint2* p = reinterpret_cast<const uint2*>(A + (long long)row * K);
+    uint32_t* o = reinterpret_cast<uint32_t*>(aq + (long long)row * K);
+    for (int i = lane; i < K / 4; i += 64) {
+        const uint2 v = p[i];
+        o[i] = pack_fp8x4(__uint_as_float(v.x << 16) * inv, __uint_as_float(v.x & 0xffff0000u) * inv, __uint_as_float(v.y << 16) * inv,
+                          __uint_as_float(v.y & 0xffff0000u) * inv);
+    }
+    __builtin_amdgcn_wave_barrier();  // every lane has read amax[row] before lane 0 replaces it
+    if (lane == 0) amax[row] = s;
+}
+// column n of a (K,N) fp32 weight: amax[n] = max_k |W[k][n]|; one thread per column, rows walked together so reads stay coalesced
+__global__ void __launch_bounds__(256) col_amax_f32_kernel(const float* __restrict__ W, float* __restrict__ amax, int K, int N) {
+    const int n = blockIdx.x * 256 + threadIdx.x;
+    if (n >= N) return;
+    float mx = 0.f;
+    for (int k = 0; k < K; k++) mx = fmaxf(mx, fabsf(W[(long long)k * N + n]));
+    amax[n] = mx;
+}
+// (K,N) fp32 -> (N,K) fp8 through a 32x33 LDS tile, each column divided by its factor s[n] = amax[n] / 448
+__global__ void __launch_bounds__(256) pack_weight_fp8_kernel(const float* __restrict__ W, uint8_t* __restrict__ out, const float* __restrict__ amax, int K,
+                                                              int N) {
+    __shared__ float tile[32][33];
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+    const int n0 = blockIdx.x * 32, k0 = blockIdx.y * 32;
+    for (int r = ty; r < 32; r += 8) {
+        const int k = k0 + r, n = n0 + tx;
+        float v = 0.f;
+        if (k < K && n < N) {
+            const float mx = amax[n];
+            v = W[(long long)k * N + n] * (mx > 0.f ? FP8_MAX / mx : 1.0f);
+        }
+        tile[r][tx] = v;
+    }
+    __syncthreads();
+    // 8 threads per output row (n), 4 consecutive k each
+    const int r = threadIdx.x >> 3, k4 = (threadIdx.x & 7) * 4;
+    const int n = n0 + r, k = k0 + k4;
+    if (n < N && k < K) *reinterpret_cast<uint32_t*>(out + (long long)n * K + k) = pack_fp8x4(tile[k4][r], tile[k4 + 1][r], tile[k4 + 2][r], tile[k4 + 3][r]);
+}
+__global__ void __launch_bounds__(256) amax_to_scale_kernel(float* __restrict__ v, int n) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i < n) v[i] = v[i] > 0.f ? v[i] * (1.0f / FP8_MAX) : 1.0f;
+}
+}  // namespace
+
+int quantize_rows_fp8(const bf16_t* A, uint8_t* aq, float* scale, int M, int K, int per_tensor, hipStream_t st) {
+    if (M <= 0) return SD3_OK;
+    if (K <= 0 || K % 4) return fail(SD3_ERR_UNSUPPORTED, "quantize_rows_fp8: K=%d must be a positive multiple of 4", K);
+    hipLaunchKernelGGL(row_amax_bf16_kernel, dim3((M + 3) / 4), dim3(256), 0, st, A, scale, M, K);
+    if (per_tensor) hipLaunchKernelGGL(broadcast_max_kernel, dim3(1), dim3(1024), 0, st, scale, M);
+    hipLaunchKernelGGL(quantize_rows_fp8_kernel, dim3((M + 3) / 4), dim3(256), 0, st, A, aq, scale, M, K);
+    return launch_status("quantize_rows_fp8");
+}
+int quantize_weight_fp8(const float* W, uint8_t* wq, float* scale, int K, int N, int per_tensor, hipStream_t st) {
+    if (K <= 0 || N <= 0) return SD3_OK;
+    if (K % 4) return fail(SD3_ERR_UNSUPPORTED, "quantize_weight_fp8: K=%d must be a multiple of 4", K);
+    hipLaunchKernelGGL(col_amax_f32_kernel, dim3((N + 255) / 256), dim3(256), 0, st, W, scale, K, N);
+    if (per_tensor) hipLaunchKernelGGL(broadcast_max_kernel, dim3(1), dim3(1024), 0, st, scale, N);
+    hipLaunchKernelGGL(pack_weight_fp8_kernel, dim3((N + 31) / 32, (K + 31) / 32), dim3(256), 0, st, W, wq, scale, K, N);
+    hipLaunchKernelGGL(amax_to_scale_kernel, dim3((N + 255) / 256), dim3(256), 0, st, scale, N);
+    return launch_status("quantize_weight_fp8");
+}
+}  // namespace sd3

@@ -8,7 +8,7 @@ import os
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libsd3_hip.so")
 
-PREC_F32, PREC_BF16 = 0, 1
+PREC_F32, PREC_BF16, PREC_BF16_FP8, PREC_BF16_FP8_TENSOR = 0, 1, 2, 3
 ACT_SILU, ACT_GELU_TANH = 0, 1
 
 vp, ci, cf, cll, cs = C.c_void_p, C.c_int, C.c_float, C.c_longlong, C.c_char_p
@@ -52,6 +52,9 @@ SIGNATURES = {
     "sd3_pack_weight_bf16": [vp, vp, ci, ci, vp],
     "sd3_gemm_bf16": [vp, vp, vp, vp, ci, ci, ci, ci, vp],
     "sd3_gemm_bf16_grouped": [vp, ci, ci, ci, vp],
+    "sd3_quantize_weight_fp8": [vp, vp, vp, ci, ci, ci, vp],
+    "sd3_quantize_rows_fp8": [vp, vp, vp, ci, ci, ci, vp],
+    "sd3_gemm_fp8": [vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, vp],
     "sd3_cast_f32_to_bf16": [vp, vp, cll, vp],
     "sd3_gemm_bf16_force_tile": [ci],
     "sd3_probe_mfma_bf16": [ci, ci, vp],

@@ -10,7 +10,7 @@ import torch
 
 from . import lib as L
 
-_PREC = {"fp32": L.PREC_F32, "f32": L.PREC_F32, "bf16": L.PREC_BF16}
+_PREC = {"fp32": L.PREC_F32, "f32": L.PREC_F32, "bf16": L.PREC_BF16, "bf16+fp8": L.PREC_BF16_FP8, "bf16+fp8-tensor": L.PREC_BF16_FP8_TENSOR}
 
 
 def _p(t):
@@ -288,7 +288,7 @@ class Context:
     def synchronize(self):
         L.call("sd3_ctx_synchronize", self._h)
 
-    PROFILE_CLASSES = ("gemm", "attention", "layernorm_modulate", "adaln_linear")
+    PROFILE_CLASSES = ("gemm", "attention", "layernorm_modulate", "adaln_linear", "gemm_fp8", "fp8_quantize")
 
     def profile_begin(self):
         L.call("sd3_profile_begin", self._h)
