@@ -180,6 +180,13 @@ int sd3_profile_end(sd3_ctx* ctx, double* ms, double* work, long long* launches)
  * This is the fused form of modules.cpp:1396-1399,1420-1432 (rmsnorm_group x4, concatenate x3, attention, split). */
 int sd3_flash_attention_bf16(const void* qkv0, const void* qkv1, void* out0, void* out1, const float* rms_q0, const float* rms_k0,
                              const float* rms_q1, const float* rms_k1, int B, int T0, int T1, int num_heads, int head_dim, void* stream);
+/* The same joint attention (without the fused norm) taken apart the way the block does it when segment 0 is short and segment 1
+ * long: one launch holds the segment-1 queries over all keys and the segment-0 queries as kv_splits work items each, every item
+ * over its own run of keys; a second small kernel merges the partial results of the split (sum_s O_s 2^(m_s-M) / sum_s l_s 2^(m_s-M)).
+ * workspace: device memory of at least B * num_heads * ceil(T0/256) * kv_splits * 256 * 66 * 4 bytes. Rows of segment 1 come out
+ * bit-identical to sd3_flash_attention_bf16, rows of segment 0 equal up to the rounding of the merge. */
+int sd3_flash_attention_bf16_split(const void* qkv0, const void* qkv1, void* out0, void* out1, int B, int T0, int T1, int num_heads, int head_dim,
+                                   int kv_splits, void* workspace, long long workspace_bytes, void* stream);
 /* out(M,N) = A(M,K) @ W + bias with A bf16 row-major, W given in the reference's fp32 (K,N) layout already packed by
  * sd3_pack_weight_bf16 into `wpacked`; out bf16. K % 64 == 0 and N % 8 == 0 required. epilogue: 0 bias, 1 bias+GELU-tanh. */
 int sd3_pack_weight_bf16(const float* W, void* wpacked, int K, int N, void* stream);
@@ -223,8 +230,12 @@ int sd3_gemm_fp8(const void* aq, const float* a_scale, const void* wq, const flo
 int sd3_cast_f32_to_bf16(const float* in, void* out, long long n, void* stream);
 /* Tuning hook with no counterpart in the reference: forces the output tile of the bf16 GEMM for every later call in this
  * process. tile = 0: chosen per call from the problem sizes (the default); 128: 128x128 tiles, two workgroups per compute
- * unit; 256: 256x256 tiles, one workgroup per compute unit. Results do not depend on the choice. */
+ * unit; 256: 256x256 tiles, one workgroup per compute unit; 192: 256x192 tiles (not with the fused qk-norm epilogue). Results do
+ * not depend on the choice. */
 int sd3_gemm_bf16_force_tile(int tile);
+/* Process-wide tuning switches by name (no counterpart in the reference); results never depend on them. "gemm_bf16_tile": as
+ * sd3_gemm_bf16_force_tile. Unknown names return SD3_ERR_INVALID_ARG. */
+int sd3_tune(const char* name, int value);
 /* Measurement aid with no counterpart in the reference: the rate (in TFLOP/s) at which the device's matrix cores run the
  * bf16 instruction the GEMM and attention kernels are built on when every wavefront issues it back to back on operands held
  * in registers (no memory or LDS traffic), with all-zero operands (random_operands = 0) or random ones (1). The two differ

@@ -45,6 +45,18 @@ struct SegDev {
     int T[2];
     int Tq[2];
     int NH, nqb;  // heads, query blocks per (batch, head)
+    // kv_splits > 1: every (batch, head, query block) becomes kv_splits work items, each over its own run of key tiles, and an item
+    // writes what it has accumulated -- unnormalised O (fp32), the softmax reference and the row sum -- for attn_combine_kernel
+    int kv_splits;
+    float* part_o;   // (items, BQ, 64)
+    float* part_ml;  // (items, BQ, 2)
+};
+// One launch covers up to three independent attention problems ("sets": in a block, the joint attention of the latent queries,
+// the extra self-attention, and the few context queries split along the keys): workgroups [0, end[0]) belong to set 0, ...
+constexpr int MAX_SETS = 3;
+struct AttnSets {
+    SegDev set[MAX_SETS];
+    int end[MAX_SETS];
 };
 
 __device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 1); }
@@ -84,8 +96,11 @@ __device__ __forceinline__ void lds_wait_last4(uint2 (&a)[8]) {
 // NORM: apply the per-head RMSNorm to q and k while loading them (K then goes through registers instead of the
 // direct global->LDS path). Without it q and k are taken as they are (already normalised by the QKV GEMM epilogue).
 template <bool NORM>
-__global__ void __launch_bounds__(NW * 64, 2) flash_attn_bf16_kernel(SegDev s, float q_scale /* log2(e)/sqrt(64) */, float eps) {
+__global__ void __launch_bounds__(NW * 64, 2) flash_attn_bf16_kernel(const AttnSets sets, float q_scale /* log2(e)/sqrt(64) */, float eps) {
     __shared__ __attribute__((aligned(1024))) char smem[SMEM_BYTES];
+    const int which = (blockIdx.x >= (unsigned)sets.end[0]) + (blockIdx.x >= (unsigned)sets.end[1]);  // uniform
+    const SegDev& s = sets.set[which];
+    const int wg_first = which ? sets.end[which - 1] : 0;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: LDS destinations of the direct loads are then scalar
     const int l32 = lane & 31, lk = lane >> 5;
@@ -94,16 +109,22 @@ __global__ void __launch_bounds__(NW * 64, 2) flash_attn_bf16_kernel(SegDev s, f
 
     // ---- workgroup -> (batch, head, query block): consecutive workgroup ids go to different XCDs (each with its own L2),
     //      so the workgroups of one XCD get a contiguous run of work items; all query blocks of a head then share K/V in one L2
-    int b, h, qblk;
+    int b, h, qblk, split, item;
     {
-        const int total = gridDim.x, wg = blockIdx.x, xcd = wg % 8, local = wg / 8;
+        const int total = sets.end[which] - wg_first, wg = blockIdx.x - wg_first, xcd = wg % 8, local = wg / 8;
         const int per = (total + 7) / 8, tall = (total % 8) ? (total % 8) : 8;
-        const int t = (xcd < tall) ? xcd * per + local : tall * per + (xcd - tall) * (per - 1) + local;
+        item = (xcd < tall) ? xcd * per + local : tall * per + (xcd - tall) * (per - 1) + local;
+        split = item % s.kv_splits;
+        const int t = item / s.kv_splits;
         const int bh = t / s.nqb;
         qblk = t % s.nqb;
         b = bh / s.NH;
         h = bh % s.NH;
     }
+    // this item's run of key tiles: [kv0, kv0 + nt * BKV), the whole sequence when kv_splits == 1
+    const int nt_all = (T + BKV - 1) / BKV, nt_per = (nt_all + s.kv_splits - 1) / s.kv_splits;
+    const int kv0 = split * nt_per * BKV;
+    const int nt = min(nt_per, nt_all - split * nt_per);  // >= 1: the host chooses kv_splits so that no item is empty
 
     // ---- Q^T operands: for block qb the lane is query (q0 + 32 qb + l32); k-step ks covers d = 16 ks + 8 lk + (0..7) ----
     const int q0 = qblk * BQ + wave * QW;
@@ -180,7 +201,7 @@ __global__ void __launch_bounds__(NW * 64, 2) flash_attn_bf16_kernel(SegDev s, f
     // advance() moves the four row pointers to the tile that starts at key t0 (branches; kept out of the pipeline steps),
     // fetch_tile() issues the loads through them (straight-line; interleaved with a step's matrix instructions)
     auto advance = [&](int t0) {
-        const bool in0 = (t0 >= BKV) && (t0 + BKV <= T0), in1 = (t0 - BKV >= T0) && (t0 + BKV <= T);
+        const bool in0 = (t0 >= kv0 + BKV) && (t0 + BKV <= T0), in1 = (t0 - BKV >= max(T0, kv0)) && (t0 + BKV <= T);
         if (in0 || in1) {
             const long long step = (long long)BKV * s.ld_qkv[in1 ? 1 : 0];
 #pragma unroll
@@ -257,7 +278,6 @@ __global__ void __launch_bounds__(NW * 64, 2) flash_attn_bf16_kernel(SegDev s, f
     //      so that neither unit waits for the other inside a wavefront. Tiles live in a ring of three LDS stages: the
     //      loads of tile t+2 are issued right after the barrier that publishes tile t+1, at which point every wavefront
     //      has finished its reads of tile t-1, whose stage they overwrite. ----
-    const int nt = (T + BKV - 1) / BKV;
     f32x16_t sacc[2];   // sacc[qb]: scores of the unit of query block qb that is in the pipeline
     Frag pf[2][2];      // pf[qb][j]: its probabilities as P^T operands
     bf16x8_t kf[4];     // K fragments of the key half whose scores are being issued
@@ -363,11 +383,11 @@ __global__ void __launch_bounds__(NW * 64, 2) flash_attn_bf16_kernel(SegDev s, f
     };
 
     // prologue: tiles 0 and 1 on their way, tile 0 visible, scores of the first unit issued
-    advance(0);
+    advance(kv0);
     fetch_tile(0);
-    if (NORM) store_k_normed(0, 0);
+    if (NORM) store_k_normed(kv0, 0);
     if (nt > 1) {
-        advance(BKV);
+        advance(kv0 + BKV);
         fetch_tile(STAGE_BYTES);
         __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8) | 4);  // vmcnt(4): all but the four loads of tile 1
     } else {
@@ -375,7 +395,7 @@ __global__ void __launch_bounds__(NW * 64, 2) flash_attn_bf16_kernel(SegDev s, f
     }
     __syncthreads();
     load_k(0, 0);
-    scores(0, 0);
+    scores(0, kv0);
     int st_cur = 0, st_nxt = STAGE_BYTES, st_ld = 2 * STAGE_BYTES;  // stages of tiles t, t+1, t+2
 
     for (int t = 0; t < nt; t++) {
@@ -384,7 +404,7 @@ __global__ void __launch_bounds__(NW * 64, 2) flash_attn_bf16_kernel(SegDev s, f
         //      frees; scores of (t,0,1); then fetch K of half 1 ----
         pv(1, 0);
         load_v(st_cur, 0, 0);
-        scores(1, t * BKV);
+        scores(1, kv0 + t * BKV);
         load_k(st_cur, 1);
         inc = probs(0);
         pv(1, 1);
@@ -394,7 +414,7 @@ __global__ void __launch_bounds__(NW * 64, 2) flash_attn_bf16_kernel(SegDev s, f
         // ---- step (t, 0, 1): PV of (t,0,0); scores of (t,1,0) ----
         lds_wait_first4(vfr);
         pv(0, 0);
-        scores(0, t * BKV + 32);
+        scores(0, kv0 + t * BKV + 32);
         inc = probs(1);
         lds_wait_last4(vfr);
         pv(0, 1);
@@ -403,14 +423,14 @@ __global__ void __launch_bounds__(NW * 64, 2) flash_attn_bf16_kernel(SegDev s, f
         // ---- step (t, 1, 0): tile t+1 becomes visible and the loads of tile t+2 set off (past the end: the last tile once
         //      more, into a stage nobody reads again); PV of (t,0,1) and fetch of V of key half 1; scores of (t,1,1); then
         //      fetch K of half 0 of tile t+1 (past the last tile: stale LDS, feeding scores that are never used) ----
-        if (NORM && t + 1 < nt) store_k_normed((t + 1) * BKV, st_nxt);
+        if (NORM && t + 1 < nt) store_k_normed(kv0 + (t + 1) * BKV, st_nxt);
         __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8));  // vmcnt(0): this thread's loads of tile t+1 have landed
         __syncthreads();  // (also in the last tile: the stage the redundant loads go to must not be in use by a slower wavefront)
-        if (t + 2 < nt) advance((t + 2) * BKV);
+        if (t + 2 < nt) advance(kv0 + (t + 2) * BKV);
         fetch_tile(st_ld);
         pv(1, 0);
         load_v(st_cur, 1, 0);
-        scores(1, t * BKV + 32);
+        scores(1, kv0 + t * BKV + 32);
         load_k(st_nxt, 0);
         inc = probs(0);
         pv(1, 1);
@@ -420,7 +440,7 @@ __global__ void __launch_bounds__(NW * 64, 2) flash_attn_bf16_kernel(SegDev s, f
         // ---- step (t, 1, 1): PV of (t,1,0); scores of (t+1,0,0) ----
         lds_wait_first4(vfr);
         pv(0, 0);
-        scores(0, t * BKV + BKV);
+        scores(0, kv0 + t * BKV + BKV);
         inc = probs(1);
         lds_wait_last4(vfr);
         pv(0, 1);
@@ -435,6 +455,22 @@ __global__ void __launch_bounds__(NW * 64, 2) flash_attn_bf16_kernel(SegDev s, f
     pv(1, 1);
     __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8));  // the redundant loads issued past the last tile have landed before LDS is reused
 
+    // ---- an item of a split: leave the unnormalised accumulators, the reference and the row sum for the combining kernel ----
+    if (s.kv_splits > 1) {
+#pragma unroll
+        for (int qb = 0; qb < 2; qb++) {
+            const long long prow = (long long)item * BQ + wave * QW + qb * 32 + l32;
+            const float l_tot = l_run[qb] + __shfl_xor(l_run[qb], 32, 64);
+            if (lk == 0) *reinterpret_cast<float2*>(s.part_ml + prow * 2) = make_float2(m_run[qb], l_tot);
+#pragma unroll
+            for (int db = 0; db < 2; db++)
+#pragma unroll
+                for (int g = 0; g < 4; g++)
+                    *reinterpret_cast<float4*>(s.part_o + prow * HS + db * 32 + 8 * g + 4 * lk) =
+                        make_float4(oacc[db][qb][4 * g + 0], oacc[db][qb][4 * g + 1], oacc[db][qb][4 * g + 2], oacc[db][qb][4 * g + 3]);
+        }
+        return;
+    }
     // ---- normalise; transpose through LDS (each wavefront its own 64-row region) so that rows leave as 16-byte stores ----
     __syncthreads();
     bf16_t* Ow = reinterpret_cast<bf16_t*>(smem) + wave * QW * O_PITCH;
@@ -471,15 +507,41 @@ __global__ void __launch_bounds__(NW * 64, 2) flash_attn_bf16_kernel(SegDev s, f
     }
 }
 
-}  // namespace
+// Merges the kv_splits partial results of every query of a split set, in split order: with M = max_s m_s,
+// out = sum_s O_s 2^(m_s - M) / sum_s l_s 2^(m_s - M). 16 lanes per query row, 4 of the 64 output values each.
+__global__ void __launch_bounds__(256) attn_combine_kernel(const SegDev s, int B) {
+    const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+    const int sub = (int)(idx & 15);
+    const long long r = idx >> 4;  // (batch, head, query block, row in block)
+    const long long rows = (long long)B * s.NH * s.nqb * BQ;
+    if (r >= rows) return;
+    const int row = (int)(r % BQ);
+    const long long t = r / BQ;  // (batch, head, query block)
+    const int qblk = (int)(t % s.nqb);
+    const long long bh = t / s.nqb;
+    const int b = (int)(bh / s.NH), h = (int)(bh % s.NH);
+    const int q = qblk * BQ + row, Tq0 = s.Tq[0];
+    if (q >= s.Tq[0] + s.Tq[1]) return;
+    const int seg = (q < Tq0) ? 0 : 1;
+    if (!s.out[seg]) return;
+    float mmax = -3.0e38f;
+    for (int k = 0; k < s.kv_splits; k++) mmax = fmaxf(mmax, s.part_ml[((t * s.kv_splits + k) * BQ + row) * 2]);
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    float l = 0.f;
+    for (int k = 0; k < s.kv_splits; k++) {
+        const long long prow = (t * s.kv_splits + k) * BQ + row;
+        const float2 ml = *reinterpret_cast<const float2*>(s.part_ml + prow * 2);
+        const float w = __builtin_amdgcn_exp2f(ml.x - mmax);
+        const float4 o = *reinterpret_cast<const float4*>(s.part_o + prow * HS + sub * 4);
+        acc.x = fmaf(o.x, w, acc.x); acc.y = fmaf(o.y, w, acc.y); acc.z = fmaf(o.z, w, acc.z); acc.w = fmaf(o.w, w, acc.w);
+        l = fmaf(ml.y, w, l);
+    }
+    const float inv = 1.0f / l;
+    bf16_t* op = s.out[seg] + ((long long)b * s.Tq[seg] + (seg ? q - Tq0 : q)) * s.ld_out[seg] + h * HS + sub * 4;
+    *reinterpret_cast<uint2*>(op) = make_uint2(pack_bf16x2(acc.x * inv, acc.y * inv), pack_bf16x2(acc.z * inv, acc.w * inv));
+}
 
-int attention_bf16(const AttnSegments& a, int B, int NH, int hs, hipStream_t st) {
-    const int T = a.T[0] + a.T[1], TQ = a.Tq[0] + a.Tq[1];
-    if (B <= 0 || NH <= 0 || TQ <= 0) return SD3_OK;
-    if (hs != HS) return fail(SD3_ERR_UNSUPPORTED, "attention (bf16): head_dim must be 64 (got %d)", hs);
-    if (T <= 0) return fail(SD3_ERR_INVALID_ARG, "attention: no keys");
-    SegDev s;
-    bool norm = false;
+int fill_set(const AttnSegments& a, int NH, SegDev& s, bool& norm) {
     for (int i = 0; i < 2; i++) {
         s.q[i] = (const bf16_t*)a.q[i]; s.k[i] = (const bf16_t*)a.k[i]; s.v[i] = (const bf16_t*)a.v[i]; s.out[i] = (bf16_t*)a.out[i];
         s.rms_q[i] = a.rms_q[i]; s.rms_k[i] = a.rms_k[i];
@@ -494,12 +556,73 @@ int attention_bf16(const AttnSegments& a, int B, int NH, int hs, hipStream_t st)
         }
     }
     s.NH = NH;
-    s.nqb = (TQ + BQ - 1) / BQ;
-    const float q_scale = 1.4426950408889634f / sqrtf((float)HS);
-    dim3 grid((unsigned)(s.nqb * NH * B)), block(NW * 64);
-    if (norm) hipLaunchKernelGGL(flash_attn_bf16_kernel<true>, grid, block, 0, st, s, q_scale, 1e-6f);
-    else hipLaunchKernelGGL(flash_attn_bf16_kernel<false>, grid, block, 0, st, s, q_scale, 1e-6f);
-    return launch_status("flash_attention_bf16");
+    s.nqb = (a.Tq[0] + a.Tq[1] + BQ - 1) / BQ;
+    s.kv_splits = 1;
+    s.part_o = nullptr;
+    s.part_ml = nullptr;
+    return SD3_OK;
 }
+
+}  // namespace
+
+// Key splits for the context queries of a joint attention, or 0 when the one-set launch is the better choice. The joint sequence
+// of the headline shape has 17 query blocks of 256 per (batch, head), the last one holding the 154 leftover rows: 816 workgroups,
+// which run as long as 1024 would (two per compute unit: 512 at a time). With the latent queries alone the count is 768, whose
+// last 256 have a compute unit to themselves and finish early; the context queries then go, split four ways along the keys into
+// short work items, into the slots those leave free, and a small kernel merges their partial results.
+int attention_bf16_context_splits(int Tc, int Tx) {
+    const int nt_all = (Tc + Tx + BKV - 1) / BKV;
+    if (Tc <= 0 || Tc > BQ || Tx < 4 * BQ || nt_all < 16) return 0;
+    return 4;
+}
+size_t attention_bf16_split_workspace_floats(int B, int NH, int Tc, int splits) {
+    const size_t items = (size_t)B * NH * ((Tc + BQ - 1) / BQ) * splits;
+    return items * BQ * (HS + 2);
+}
+
+int attention_bf16_multi(const AttnSegments* jobs, const int* kv_splits, float* const* split_ws, int n, int B, int NH, int hs, hipStream_t st) {
+    if (n < 1 || n > MAX_SETS) return fail(SD3_ERR_INVALID_ARG, "attention: 1 to %d sets per launch (got %d)", MAX_SETS, n);
+    if (hs != HS) return fail(SD3_ERR_UNSUPPORTED, "attention (bf16): head_dim must be 64 (got %d)", hs);
+    if (B <= 0 || NH <= 0) return SD3_OK;
+    AttnSets sets{};
+    bool norm = false;
+    int m = 0, total = 0;
+    for (int i = 0; i < n; i++) {
+        const AttnSegments& a = jobs[i];
+        const int T = a.T[0] + a.T[1], TQ = a.Tq[0] + a.Tq[1];
+        if (TQ <= 0) continue;
+        if (T <= 0) return fail(SD3_ERR_INVALID_ARG, "attention: no keys");
+        SegDev& s = sets.set[m];
+        SD3_TRY(fill_set(a, NH, s, norm));
+        const int S = kv_splits ? kv_splits[i] : 1;
+        if (S > 1) {
+            const int nt_all = (T + BKV - 1) / BKV, per = (nt_all + S - 1) / S;
+            if (per * (S - 1) >= nt_all) return fail(SD3_ERR_INVALID_ARG, "attention: %d key splits leave an empty one for %d keys", S, T);
+            if (!split_ws || !split_ws[i]) return fail(SD3_ERR_INVALID_ARG, "attention: a split set needs its workspace");
+            s.kv_splits = S;
+            s.part_o = split_ws[i];
+            s.part_ml = split_ws[i] + (size_t)B * NH * s.nqb * S * BQ * HS;
+        }
+        total += s.nqb * NH * B * s.kv_splits;
+        sets.end[m++] = total;
+    }
+    if (m == 0) return SD3_OK;
+    for (int i = m; i < MAX_SETS; i++) sets.end[i] = total;
+    const float q_scale = 1.4426950408889634f / sqrtf((float)HS);
+    dim3 grid((unsigned)total), block(NW * 64);
+    if (norm) hipLaunchKernelGGL(flash_attn_bf16_kernel<true>, grid, block, 0, st, sets, q_scale, 1e-6f);
+    else hipLaunchKernelGGL(flash_attn_bf16_kernel<false>, grid, block, 0, st, sets, q_scale, 1e-6f);
+    SD3_TRY(launch_status("flash_attention_bf16"));
+    for (int i = 0; i < m; i++) {
+        const SegDev& s = sets.set[i];
+        if (s.kv_splits <= 1) continue;
+        const long long threads = (long long)B * NH * s.nqb * BQ * 16;
+        hipLaunchKernelGGL(attn_combine_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st, s, B);
+        SD3_TRY(launch_status("attention_combine"));
+    }
+    return SD3_OK;
+}
+
+int attention_bf16(const AttnSegments& a, int B, int NH, int hs, hipStream_t st) { return attention_bf16_multi(&a, nullptr, nullptr, 1, B, NH, hs, st); }
 
 }  // namespace sd3

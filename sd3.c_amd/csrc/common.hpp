@@ -205,5 +205,12 @@ struct AttnSegments {
 };
 int attention_f32(const AttnSegments& s, int B, int NH, int HS, hipStream_t st);
 int attention_bf16(const AttnSegments& s, int B, int NH, int HS, hipStream_t st);
+// Up to three attention problems in one launch. kv_splits[i] > 1 (or null: all 1) splits the keys of set i into that many runs, one
+// work item each, whose partial results go through split_ws[i] (attention_bf16_split_workspace_floats floats) and are merged by a
+// second, small kernel. attention_bf16_context_splits: the number of splits that pays for the Tc context queries of a joint
+// attention next to Tx latent ones, or 0 when the plain one-set launch is the better choice.
+int attention_bf16_multi(const AttnSegments* sets, const int* kv_splits, float* const* split_ws, int n, int B, int NH, int HS, hipStream_t st);
+int attention_bf16_context_splits(int Tc, int Tx);
+size_t attention_bf16_split_workspace_floats(int B, int NH, int Tc, int splits);
 
 }  // namespace sd3

@@ -242,6 +242,11 @@ size_t block_workspace_bytes(const Dims& d, int prec) {
     act(mc * 3 * d.C); act(mx * 3 * d.C);                  // c_qkv, x_qkv
     if (d.dual) act(mx * 3 * d.C);                         // x_qkv2
     act(mc * d.C); act(mx * d.C);                          // c_att, x_att
+    if (is_bf(prec)) {
+        if (d.dual) act(mx * d.C);                         // x_att2: both attentions of a dual block run in one launch
+        const int S = attention_bf16_context_splits(d.Tc, d.Tx);
+        if (S) b.take<float>(attention_bf16_split_workspace_floats(d.B, d.NH, d.Tc, S));
+    }
     act(mc * d.E * d.C); act(mx * d.E * d.C);              // c_mlp, x_mlp
     b.take<float>((size_t)d.B * 6 * d.C); b.take<float>((size_t)d.B * 9 * d.C);  // ada_c, ada_x
     return b.off;
@@ -365,6 +370,13 @@ int run_block(sd3_ctx* ctx, int prec, const float* y, float* c, float* x, const 
     void* x_qkv2 = d.dual ? act((size_t)mx * 3 * C) : nullptr;  // q,k,v of the extra self-attention branch
     void* c_att = act((size_t)mc * C);
     void* x_att = act((size_t)mx * C);
+    void* x_att2 = x_att;  // output of the extra self-attention (bf16 path: a buffer of its own, the two attentions share a launch)
+    float* split_ws = nullptr;
+    const int ctx_splits = is_bf(prec) ? attention_bf16_context_splits(Tc, Tx) : 0;
+    if (is_bf(prec)) {
+        if (d.dual) x_att2 = act((size_t)mx * C);
+        if (ctx_splits) split_ws = ws.take<float>(attention_bf16_split_workspace_floats(B, d.NH, Tc, ctx_splits));
+    }
     void* c_mlp = act((size_t)mc * d.E * C);
     void* x_mlp = act((size_t)mx * d.E * C);
     float* ada_c_buf = ws.take<float>((size_t)B * 6 * C);
@@ -429,13 +441,49 @@ int run_block(sd3_ctx* ctx, int prec, const float* y, float* c, float* x, const 
         SD3_TRY(rmsnorm_rows((float*)x_qkv, (float*)x_qkv, w.x_rms_q, nullptr, 1e-6f, mx, d.NH, d.HS, 3 * C, 3 * C, st));
         SD3_TRY(rmsnorm_rows((float*)seg_ptr(x_qkv, 1), (float*)seg_ptr(x_qkv, 1), w.x_rms_k, nullptr, 1e-6f, mx, d.NH, d.HS, 3 * C, 3 * C, st));
     }
-    {
-        AttnSegments a{};
-        a.q[0] = c_qkv; a.k[0] = seg_ptr(c_qkv, 1); a.v[0] = seg_ptr(c_qkv, 2); a.out[0] = d.discard ? nullptr : c_att;
-        a.q[1] = x_qkv; a.k[1] = seg_ptr(x_qkv, 1); a.v[1] = seg_ptr(x_qkv, 2); a.out[1] = x_att;
-        a.ld_qkv[0] = a.ld_qkv[1] = 3 * C; a.ld_out[0] = a.ld_out[1] = C;
-        a.T[0] = a.Tq[0] = Tc; a.T[1] = a.Tq[1] = Tx;
-        SD3_TRY(attention(ctx, a, B, d.NH, d.HS, bf));  // q and k arrive normalised on both paths
+    AttnSegments joint{}, dual_set{};
+    joint.q[0] = c_qkv; joint.k[0] = seg_ptr(c_qkv, 1); joint.v[0] = seg_ptr(c_qkv, 2); joint.out[0] = d.discard ? nullptr : c_att;
+    joint.q[1] = x_qkv; joint.k[1] = seg_ptr(x_qkv, 1); joint.v[1] = seg_ptr(x_qkv, 2); joint.out[1] = x_att;
+    joint.ld_qkv[0] = joint.ld_qkv[1] = 3 * C; joint.ld_out[0] = joint.ld_out[1] = C;
+    joint.T[0] = joint.Tq[0] = Tc; joint.T[1] = joint.Tq[1] = Tx;
+    if (d.dual) {  // extra self-attention over the latent tokens (modules.cpp:1440-1453): independent of the joint one
+        dual_set.q[0] = x_qkv2; dual_set.k[0] = seg_ptr(x_qkv2, 1); dual_set.v[0] = seg_ptr(x_qkv2, 2); dual_set.out[0] = x_att2;
+        dual_set.ld_qkv[0] = dual_set.ld_qkv[1] = 3 * C; dual_set.ld_out[0] = dual_set.ld_out[1] = C;
+        dual_set.T[0] = dual_set.Tq[0] = Tx;
+    }
+    if (bf) {
+        // One launch for everything attention has to do in this block. With few context tokens beside many latent ones the joint
+        // attention is taken apart by queries: the latent queries as one set, the context queries as short work items split along
+        // the keys (see attention_bf16_context_splits), the extra self-attention as a third set.
+        AttnSegments sets[3];
+        int splits[3] = {1, 1, 1};
+        float* wsp[3] = {nullptr, nullptr, nullptr};
+        int n = 0;
+        double flop = 0;
+        const double Tj = (double)Tc + Tx;
+        if (ctx_splits) {
+            sets[n] = joint;
+            sets[n].Tq[0] = 0; sets[n].out[0] = nullptr;
+            n++;
+        } else {
+            sets[n++] = joint;
+        }
+        flop += 4.0 * B * d.NH * Tj * Tj * d.HS;
+        if (d.dual) {
+            sets[n++] = dual_set;
+            flop += 4.0 * B * d.NH * (double)Tx * Tx * d.HS;
+        }
+        if (ctx_splits && !d.discard) {
+            sets[n] = joint;
+            sets[n].Tq[1] = 0; sets[n].out[1] = nullptr;
+            splits[n] = ctx_splits;
+            wsp[n] = split_ws;
+            n++;
+        }
+        ProfScope ps(ctx, SD3_PROF_ATTENTION, flop, 1);
+        SD3_TRY(attention_bf16_multi(sets, splits, wsp, n, B, d.NH, d.HS, st));  // q and k arrive normalised
+    } else {
+        SD3_TRY(attention(ctx, joint, B, d.NH, d.HS, bf));
     }
     // ---- out-projections with the gate and the residual add in the epilogue (modules.cpp:1435-1436, 1459-1462, 1481-1485)
     GemmEpilogueArgs gx, gc;
@@ -452,14 +500,10 @@ int run_block(sd3_ctx* ctx, int prec, const float* y, float* c, float* x, const 
             SD3_TRY(rmsnorm_rows((float*)x_qkv2, (float*)x_qkv2, w.x2_rms_q, nullptr, 1e-6f, mx, d.NH, d.HS, 3 * C, 3 * C, st));
             SD3_TRY(rmsnorm_rows((float*)seg_ptr(x_qkv2, 1), (float*)seg_ptr(x_qkv2, 1), w.x2_rms_k, nullptr, 1e-6f, mx, d.NH, d.HS, 3 * C, 3 * C, st));
         }
-        AttnSegments a{};
-        a.q[0] = x_qkv2; a.k[0] = seg_ptr(x_qkv2, 1); a.v[0] = seg_ptr(x_qkv2, 2); a.out[0] = x_att;
-        a.ld_qkv[0] = a.ld_qkv[1] = 3 * C; a.ld_out[0] = a.ld_out[1] = C;
-        a.T[0] = a.Tq[0] = Tx;
-        SD3_TRY(attention(ctx, a, B, d.NH, d.HS, bf));
+        if (!bf) SD3_TRY(attention(ctx, dual_set, B, d.NH, d.HS, bf));
         GemmEpilogueArgs g2;
         g2.rows_per_batch = Tx; g2.gate = xchunk(8); g2.gate_ld = ldx_ada; g2.resid = x;
-        SD3_TRY(linear_layer(ctx, prec, x_att, w.x2_out_w, w.x2_out_b, x, 1, C, mx, C, C, EPI_GATE_RESID, g2));
+        SD3_TRY(linear_layer(ctx, prec, x_att2, w.x2_out_w, w.x2_out_b, x, 1, C, mx, C, C, EPI_GATE_RESID, g2));
     }
 
     // ---- MLPs of both streams (modules.cpp:1463-1476, 1488-1504)
@@ -1148,6 +1192,33 @@ int sd3_flash_attention_bf16(const void* qkv0, const void* qkv1, void* out0, voi
     }
     return attention_bf16(a, B, num_heads, head_dim, ST(stream));
 }
+int sd3_flash_attention_bf16_split(const void* qkv0, const void* qkv1, void* out0, void* out1, int B, int T0, int T1, int num_heads, int head_dim,
+                                   int kv_splits, void* workspace, long long workspace_bytes, void* stream) {
+    SD3_REQUIRE(B >= 0 && T0 > 0 && T1 > 0 && num_heads > 0 && head_dim > 0 && kv_splits >= 2, "flash_attention_bf16_split: bad sizes");
+    if (B == 0) return SD3_OK;
+    NOTNULL(qkv0); NOTNULL(qkv1); NOTNULL(out0); NOTNULL(out1); NOTNULL(workspace);
+    const long long need = (long long)attention_bf16_split_workspace_floats(B, num_heads, T0, kv_splits) * (long long)sizeof(float);
+    SD3_REQUIRE(workspace_bytes >= need, "flash_attention_bf16_split: the workspace holds %lld bytes, %lld are needed", workspace_bytes, need);
+    const int C = num_heads * head_dim;
+    AttnSegments joint{};
+    const void* qkv[2] = {qkv0, qkv1};
+    void* outs[2] = {out0, out1};
+    const int T[2] = {T0, T1};
+    for (int i = 0; i < 2; i++) {
+        joint.q[i] = qkv[i];
+        joint.k[i] = (const char*)qkv[i] + (size_t)C * 2;
+        joint.v[i] = (const char*)qkv[i] + (size_t)2 * C * 2;
+        joint.out[i] = outs[i];
+        joint.ld_qkv[i] = 3 * C; joint.ld_out[i] = C;
+        joint.T[i] = joint.Tq[i] = T[i];
+    }
+    AttnSegments sets[2] = {joint, joint};
+    sets[0].Tq[0] = 0; sets[0].out[0] = nullptr;  // the segment-1 queries, whole key range
+    sets[1].Tq[1] = 0; sets[1].out[1] = nullptr;  // the segment-0 queries, split along the keys
+    const int splits[2] = {1, kv_splits};
+    float* wsp[2] = {nullptr, (float*)workspace};
+    return attention_bf16_multi(sets, splits, wsp, 2, B, num_heads, head_dim, ST(stream));
+}
 int sd3_pack_weight_bf16(const float* W, void* wpacked, int K, int N, void* stream) {
     SD3_REQUIRE(K > 0 && N > 0, "pack_weight_bf16: bad sizes");
     NOTNULL(W); NOTNULL(wpacked);
@@ -1208,6 +1279,11 @@ int sd3_gemm_fp8(const void* aq, const float* a_scale, const void* wq, const flo
     GemmBf16Problem q{(const bf16_t*)aq, (const bf16_t*)wq, out, N, M, N, K, GemmEpilogueArgs{}};
     q.ea.bias = bias; q.ea.a_scale = a_scale; q.ea.w_scale = w_scale;
     return gemm_fp8_grouped(&q, 1, out_is_f32, epilogue, ST(stream));
+}
+int sd3_tune(const char* name, int value) {
+    NOTNULL(name);
+    if (!std::strcmp(name, "gemm_bf16_tile")) return sd3_gemm_bf16_force_tile(value);
+    return fail(SD3_ERR_INVALID_ARG, "sd3_tune: unknown setting '%s'", name);
 }
 int sd3_cast_f32_to_bf16(const float* in, void* out, long long n, void* stream) {
     SD3_REQUIRE(n >= 0, "cast: negative size");

@@ -49,6 +49,7 @@ SIGNATURES = {
     "sd3_profile_begin": [vp],
     "sd3_profile_end": [vp, vp, vp, vp],
     "sd3_flash_attention_bf16": [vp] * 8 + [ci] * 5 + [vp],
+    "sd3_flash_attention_bf16_split": [vp] * 4 + [ci] * 6 + [vp, cll, vp],
     "sd3_pack_weight_bf16": [vp, vp, ci, ci, vp],
     "sd3_gemm_bf16": [vp, vp, vp, vp, ci, ci, ci, ci, vp],
     "sd3_gemm_bf16_grouped": [vp, ci, ci, ci, vp],
@@ -57,6 +58,7 @@ SIGNATURES = {
     "sd3_gemm_fp8": [vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, ci, vp],
     "sd3_cast_f32_to_bf16": [vp, vp, cll, vp],
     "sd3_gemm_bf16_force_tile": [ci],
+    "sd3_tune": [cs, ci],
     "sd3_probe_mfma_bf16": [ci, ci, vp],
 }
 

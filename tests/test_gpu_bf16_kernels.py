@@ -57,6 +57,41 @@ def test_flash_attention_bf16(B, T0, T1, NH):
     assert float((got - ref).abs().max()) <= 0.05  # outputs are O(1) convex combinations of N(0,1) values
 
 
+@pytest.mark.parametrize("B,T0,T1,NH,S", [(2, 154, 4096, 24, 4), (1, 77, 1100, 3, 4), (1, 1, 130, 2, 2), (2, 200, 600, 2, 3), (1, 256, 64, 1, 5)])
+def test_flash_attention_bf16_taken_apart_by_queries_with_key_splits(B, T0, T1, NH, S):
+    """What the block does at the headline shape (first case): latent queries in one set, the context queries split along the keys and
+    merged by the combining kernel. Latent rows must equal the one-set kernel bit for bit; context rows agree with it and with fp32
+    arithmetic to bf16 rounding."""
+    HS, C = 64, NH * 64
+    g = torch.Generator(device="cuda").manual_seed(T0 * 3 + T1 + S)
+    qkv0 = torch.randn((B * T0, 3 * C), device="cuda", generator=g).bfloat16()
+    qkv1 = torch.randn((B * T1, 3 * C), device="cuda", generator=g).bfloat16()
+    ref0 = torch.zeros((B * T0, C), device="cuda", dtype=torch.bfloat16)
+    ref1 = torch.zeros((B * T1, C), device="cuda", dtype=torch.bfloat16)
+    L.call("sd3_flash_attention_bf16", qkv0.data_ptr(), qkv1.data_ptr(), ref0.data_ptr(), ref1.data_ptr(), None, None, None, None, B, T0, T1, NH, HS, None)
+    out0, out1 = torch.zeros_like(ref0), torch.zeros_like(ref1)
+    ws = torch.empty(B * NH * ((T0 + 255) // 256) * S * 256 * 66, device="cuda")
+    ws.fill_(float("nan"))  # whatever is read must have been written by this call
+    L.call("sd3_flash_attention_bf16_split", qkv0.data_ptr(), qkv1.data_ptr(), out0.data_ptr(), out1.data_ptr(), B, T0, T1, NH, HS, S, ws.data_ptr(),
+           ws.numel() * 4, None)
+    torch.cuda.synchronize()
+    assert torch.equal(out1, ref1)
+    assert torch.isfinite(out0.float()).all()
+    assert float((out0.float() - ref0.float()).abs().max()) <= 0.03  # two bf16 roundings of O(1) values apart at most
+    # fp32 softmax(q k^T / 8) v for the context queries over the joint keys (no norm in this call)
+    q0, k0, v0 = qkv0.float().view(B, T0, 3, NH, HS).unbind(2)
+    _, k1, v1 = qkv1.float().view(B, T1, 3, NH, HS).unbind(2)
+    k, v = torch.cat([k0, k1], 1), torch.cat([v0, v1], 1)
+    p = torch.softmax(torch.einsum("bqhd,bkhd->bhqk", q0, k) / 8.0, -1)
+    naive = torch.einsum("bhqk,bkhd->bqhd", p, v).reshape(B * T0, C)
+    assert rel_l2(host(out0), host(naive)) <= 1e-2
+    with pytest.raises(L.Sd3Error):  # more splits than key tiles
+        L.call("sd3_flash_attention_bf16_split", qkv0.data_ptr(), qkv1.data_ptr(), out0.data_ptr(), out1.data_ptr(), B, T0, T1, NH, HS, 4096, ws.data_ptr(),
+               1 << 40, None)
+    with pytest.raises(L.Sd3Error):  # workspace too small
+        L.call("sd3_flash_attention_bf16_split", qkv0.data_ptr(), qkv1.data_ptr(), out0.data_ptr(), out1.data_ptr(), B, T0, T1, NH, HS, S, ws.data_ptr(), 16, None)
+
+
 def test_flash_attention_bf16_without_qk_norm_and_ones_v():
     B, T0, T1, NH, HS = 1, 10, 200, 2, 64
     C = NH * HS
