@@ -570,10 +570,12 @@ int fill_set(const AttnSegments& a, int NH, SegDev& s, bool& norm) {
 // which run as long as 1024 would (two per compute unit: 512 at a time). With the latent queries alone the count is 768, whose
 // last 256 have a compute unit to themselves and finish early; the context queries then go, split four ways along the keys into
 // short work items, into the slots those leave free, and a small kernel merges their partial results.
+int g_attention_context_splits = -1;  // -1: chosen from the sizes; 0: never split; n >= 2: n splits wherever splitting applies (sd3_tune)
 int attention_bf16_context_splits(int Tc, int Tx) {
     const int nt_all = (Tc + Tx + BKV - 1) / BKV;
-    if (Tc <= 0 || Tc > BQ || Tx < 4 * BQ || nt_all < 16) return 0;
-    return 4;
+    if (Tc <= 0 || Tc > BQ || Tx < 4 * BQ || nt_all < 16 || g_attention_context_splits == 0) return 0;
+    const int want = g_attention_context_splits > 0 ? g_attention_context_splits : 4;
+    return want < 2 ? 2 : (want > 8 ? 8 : want);
 }
 size_t attention_bf16_split_workspace_floats(int B, int NH, int Tc, int splits) {
     const size_t items = (size_t)B * NH * ((Tc + BQ - 1) / BQ) * splits;

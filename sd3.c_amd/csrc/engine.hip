@@ -33,6 +33,11 @@ const char* last_error() { return g_err; }
 
 using namespace sd3;
 
+namespace sd3 {
+extern int g_attention_context_splits;  // attention_bf16.hip
+extern int g_gemm_bf16_row_split;       // gemm_bf16.hip
+}
+
 // ------------------------------------------------------------------ fixed scratch of the entry point that allocates nothing
 // Lives in device memory from the moment the code object is loaded on a device until the process ends; every device has
 // its own copy at its own address. Host code never uses the array's name as an address: the address on a device is asked
@@ -1283,6 +1288,15 @@ int sd3_gemm_fp8(const void* aq, const float* a_scale, const void* wq, const flo
 int sd3_tune(const char* name, int value) {
     NOTNULL(name);
     if (!std::strcmp(name, "gemm_bf16_tile")) return sd3_gemm_bf16_force_tile(value);
+    if (!std::strcmp(name, "gemm_bf16_row_split")) {
+        g_gemm_bf16_row_split = value != 0;
+        return SD3_OK;
+    }
+    if (!std::strcmp(name, "attention_context_splits")) {
+        SD3_REQUIRE(value >= -1 && value != 1 && value <= 8, "sd3_tune(%s): -1 (automatic), 0 (off) or 2..8 (got %d)", name, value);
+        g_attention_context_splits = value;
+        return SD3_OK;
+    }
     return fail(SD3_ERR_INVALID_ARG, "sd3_tune: unknown setting '%s'", name);
 }
 int sd3_cast_f32_to_bf16(const float* in, void* out, long long n, void* stream) {

@@ -570,6 +570,7 @@ int launch_epi(int variant, ProbSet& args, int n, hipStream_t st) {
 }  // namespace
 
 std::atomic<long long> g_gemm_bf16_launches{0};
+int g_gemm_bf16_row_split = 1;  // 0: never split a problem's rows over two launches (sd3_tune)
 int g_gemm_bf16_variant = -1;  // -1: choose by shape; 0 / 4: forced 128x128 / 256x256 tiles (sd3_gemm_bf16_force_tile); 1: 128x128 with a ring of four stages
 
 static int grouped_impl(const GemmBf16Problem* probs, int n, int out_is_f32, int epi, bool fp8, hipStream_t st) {
@@ -655,6 +656,30 @@ static int grouped_impl(const GemmBf16Problem* probs, int n, int out_is_f32, int
         const double apart256 = rounds(big256, cus) + SMALL_LAUNCH, apart128 = ROUND128 * rounds(big128, 2 * cus) + SMALL_LAUNCH;
         if (apart256 < best) { best = apart256; plan = 2; }
         if (apart128 < best) { best = apart128; plan = 3; }
+    }
+    // One more plan for a single many-row problem whose 256x256 tiles fill R >= 1 rounds and leave a partial one: its first rows as R
+    // full rounds of 256x256 tiles, its remaining rows together with the few-row problems as 128x128 tiles in a second launch (a
+    // round of those costs 0.62). Only for epilogues that do not look at the row index (a row split would shift the batch boundaries).
+    if (g_gemm_bf16_row_split && nb == 1 && !fp8 && (epi == EPI_BIAS || epi == EPI_BIAS_GELU || epi == EPI_BIAS_SILU || epi == EPI_QKV_NORM)) {
+        const Prob& q = big.p[0];
+        const int tn = (q.N + 255) / 256, tm = (q.M + 255) / 256;
+        const int R = (int)(big256 / cus), m1 = R > 0 ? (R * cus) / tn : 0;  // row tiles that fit R full rounds
+        if (R > 0 && m1 > 0 && m1 < tm) {
+            Prob head = q, tail = q;
+            head.M = m1 * 256;
+            tail.M = q.M - head.M;
+            tail.A = q.A + (long long)head.M * q.K;
+            tail.out = (char*)q.out + (long long)head.M * q.ldc * (out_is_f32 ? 4 : 2);
+            const double split = rounds(tiles(head, 256), cus) + ROUND128 * rounds(tiles(tail, 128) + small128, 2 * cus);
+            if (split < best) {
+                ProbSet first{}, second{};
+                first.p[0] = head;
+                second.p[0] = tail;
+                for (int i = 0; i < ns; i++) second.p[1 + i] = small.p[i];
+                SD3_TRY(launch(first, 1, 4));
+                return launch(second, 1 + ns, 0);
+            }
+        }
     }
     if (plan >= 2) {
         SD3_TRY(launch(small, ns, v_small));
