@@ -236,8 +236,8 @@ int sd3_gemm_bf16_force_tile(int tile);
 /* Process-wide tuning switches by name (no counterpart in the reference); results never depend on them. "gemm_bf16_tile": as
  * sd3_gemm_bf16_force_tile; "attention_context_splits": -1 chosen from the sizes (default), 0 never, 2..8 that many key splits for
  * the context queries of a block's joint attention wherever splitting applies (results of those rows change in the last bf16 bit
- * with the number of splits; a workspace sized for one setting serves only that setting: set it before the first forward).
- * Unknown names return SD3_ERR_INVALID_ARG. */
+ * with the number of splits); "gemm_bf16_row_split": 0 / 1 (default), whether a many-row problem that leaves a partial round of
+ * 256x256 tiles may send its last rows to a second launch of 128x128 tiles. Unknown names return SD3_ERR_INVALID_ARG. */
 int sd3_tune(const char* name, int value);
 /* Measurement aid with no counterpart in the reference: the rate (in TFLOP/s) at which the device's matrix cores run the
  * bf16 instruction the GEMM and attention kernels are built on when every wavefront issues it back to back on operands held

@@ -158,6 +158,41 @@ __device__ __forceinline__ void gemm_tile(const Prob& pr, const int wg, char* sm
     const int l32 = lane & 31, lk = lane >> 5;   // position in a 32x32 block
     const int lr = lane & 15, lg = lane >> 4;    // position in a 16x16 block
 
+    // ---- epilogue set-up ----
+    constexpr int WNC = BN / WN;        // columns per wavefront
+    constexpr int EP = WNC + 4;         // fp32 pitch of the staging slab
+    static_assert(WM * WN * 32 * EP * 4 <= smem_bytes<BM, BN, WM, WN, STAGES>(), "epilogue staging must fit in the LDS allocation");
+    constexpr int CPR = WNC / 4;        // float4 chunks per row
+    static_assert(WNC % 4 == 0 && CPR <= 64, "a row of the wavefront's slab is made of float4 chunks");
+    // rows covered by one pass of the wavefront: the largest power of two with RPI * CPR <= 64 (when CPR does not divide 64, as with
+    // 48-column slabs, the lanes beyond RPI * CPR sit the epilogue out)
+    constexpr int RPI = CPR > 32 ? 1 : CPR > 16 ? 2 : CPR > 8 ? 4 : CPR > 4 ? 8 : CPR > 2 ? 16 : 32;
+    // rows per slab: 32 (measured faster than 16 on the 64-column slabs of the 256x256 tile), 16 for 48-column slabs
+    constexpr int SR = (M16 && WNC % 64 != 0) ? 16 : 32;
+    constexpr int NSLAB = BM / WM / SR;
+    constexpr int NP = SR / RPI;        // rows of a slab per lane
+    float* slab = reinterpret_cast<float*>(smem) + wave * 32 * EP;
+    float* outf = reinterpret_cast<float*>(out_);
+    bf16_t* outh = reinterpret_cast<bf16_t*>(out_);
+    const bool lane_on = lane < RPI * CPR;
+    const int e_row = lane_on ? lane / CPR : 0, e_col = lane_on ? (lane % CPR) * 4 : 0;
+    const int n0 = n_blk + wn * WNC + e_col;
+    const bool vec_ok = ((N & 3) == 0) && ((ldc & 3) == 0);
+    const int nvalid = lane_on ? min(4, N - n0) : 0;  // <= 0 for lanes beyond the last column (and for lanes that sit out)
+    // batch index of a row without a division per row: the tile starts in batch b0 and crosses a boundary every rpb rows
+    const int rpb = epi.rows_per_batch, b0 = m_blk / rpb;
+    // gated layers: the residual rows of the NEXT slab are requested before the current slab goes through LDS, so that
+    // their latency is not paid once per slab with nothing else to do
+    constexpr bool PREFETCH_RESID = (EPI == EPI_GATE_RESID);
+    float4 rnext[PREFETCH_RESID ? NP : 1];
+    auto request_resid = [&](int i) {
+        if (PREFETCH_RESID && vec_ok)
+#pragma unroll
+            for (int p = 0; p < NP; p++) {
+                const int m = m_blk + wm * (BM / WM) + i * SR + p * RPI + e_row;
+                if (m < M && nvalid > 0) rnext[p] = *reinterpret_cast<const float4*>(epi.resid + (long long)m * ldc + n0);
+            }
+    };
     if constexpr (M16) {
         // v_mfma_f32_16x16x32_bf16 operands: lane l holds row (column) l%16 of its block and the 8 consecutive k values 8*(l/16).. of
         // the 32-deep step: one 16-byte chunk of the row's 128-byte LDS line, chunk (4*step + l/16) ^ swz(row)
@@ -341,26 +376,6 @@ __device__ __forceinline__ void gemm_tile(const Prob& pr, const int wg, char* sm
     // 4-byte scattered stores; each wavefront instead transposes one 32-row slab at a time through its private LDS
     // region (the tile ring is free now) and leaves with 16 lanes covering 64 contiguous columns of one row.
     __syncthreads();
-    constexpr int WNC = BN / WN;        // columns per wavefront
-    constexpr int EP = WNC + 4;         // fp32 pitch of the staging slab
-    static_assert(WM * WN * 32 * EP * 4 <= smem_bytes<BM, BN, WM, WN, STAGES>(), "epilogue staging must fit in the LDS allocation");
-    constexpr int CPR = WNC / 4;        // float4 chunks per row
-    static_assert(WNC % 4 == 0 && CPR <= 64, "a row of the wavefront's slab is made of float4 chunks");
-    // rows covered by one pass of the wavefront: the largest power of two with RPI * CPR <= 64 (when CPR does not divide 64, as with
-    // 48-column slabs, the lanes beyond RPI * CPR sit the epilogue out)
-    constexpr int RPI = CPR > 32 ? 1 : CPR > 16 ? 2 : CPR > 8 ? 4 : CPR > 4 ? 8 : CPR > 2 ? 16 : 32;
-    // rows per slab: 32, or 16 where 32 would take more than four passes (the row registers of a slab are all live at once)
-    constexpr int SR = (M16 && 32 / RPI > 4) ? 16 : 32;
-    constexpr int NSLAB = BM / WM / SR;
-    constexpr int NP = SR / RPI;        // rows of a slab per lane
-    float* slab = reinterpret_cast<float*>(smem) + wave * 32 * EP;
-    float* outf = reinterpret_cast<float*>(out_);
-    bf16_t* outh = reinterpret_cast<bf16_t*>(out_);
-    const bool lane_on = lane < RPI * CPR;
-    const int e_row = lane_on ? lane / CPR : 0, e_col = lane_on ? (lane % CPR) * 4 : 0;
-    const int n0 = n_blk + wn * WNC + e_col;
-    const bool vec_ok = ((N & 3) == 0) && ((ldc & 3) == 0);
-    const int nvalid = lane_on ? min(4, N - n0) : 0;  // <= 0 for lanes beyond the last column (and for lanes that sit out)
     float bias4[4] = {0.f, 0.f, 0.f, 0.f};
     if (epi.bias)
 #pragma unroll
@@ -371,20 +386,6 @@ __device__ __forceinline__ void gemm_tile(const Prob& pr, const int wg, char* sm
 #pragma unroll
         for (int c = 0; c < 4; c++)
             if (c < nvalid) ws4[c] = epi.w_scale[n0 + c];
-    // batch index of a row without a division per row: the tile starts in batch b0 and crosses a boundary every rpb rows
-    const int rpb = epi.rows_per_batch, b0 = m_blk / rpb;
-    // gated layers: the residual rows of the NEXT slab are requested before the current slab goes through LDS, so that
-    // their latency is not paid once per slab with nothing else to do
-    constexpr bool PREFETCH_RESID = (EPI == EPI_GATE_RESID);
-    float4 rnext[PREFETCH_RESID ? NP : 1];
-    auto request_resid = [&](int i) {
-        if (PREFETCH_RESID && vec_ok)
-#pragma unroll
-            for (int p = 0; p < NP; p++) {
-                const int m = m_blk + wm * (BM / WM) + i * SR + p * RPI + e_row;
-                if (m < M && nvalid > 0) rnext[p] = *reinterpret_cast<const float4*>(epi.resid + (long long)m * ldc + n0);
-            }
-    };
     request_resid(0);
 #pragma unroll
     for (int i = 0; i < NSLAB; i++) {

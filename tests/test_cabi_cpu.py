@@ -83,6 +83,16 @@ def test_argument_errors_are_status_codes_not_exits():
         L.call("sd3_silu", None, None, 8, None)
 
 
+def test_tuning_switches_are_checked():
+    lib = L.load()
+    assert lib.sd3_tune(b"gemm_bf16_tile", 192) == 0 and lib.sd3_tune(b"gemm_bf16_tile", 0) == 0
+    assert lib.sd3_tune(b"gemm_bf16_tile", 100) == 1
+    assert lib.sd3_tune(b"attention_context_splits", 1) == 1 and lib.sd3_tune(b"attention_context_splits", -1) == 0
+    assert lib.sd3_tune(b"gemm_bf16_row_split", 1) == 0
+    assert lib.sd3_tune(b"no_such_switch", 1) == 1 and b"unknown setting" in lib.sd3_last_error()
+    assert lib.sd3_tune(None, 1) == 1
+
+
 def test_context_creation_without_a_gpu_fails_cleanly():
     import torch
     if torch.cuda.is_available():

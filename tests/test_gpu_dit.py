@@ -171,6 +171,29 @@ def test_dit_missing_parameter_is_reported():
     assert e.value.status == 2 and "linear_out.weight" in str(e.value)
 
 
+def test_forwards_on_alternating_streams_share_the_context_safely():
+    """The workspace and the derived weight copies belong to the context, not to a stream: a change of stream makes the new stream
+    wait for what was queued on the old one, so back-to-back forwards on two streams with different inputs give the results of the
+    same forwards run one at a time."""
+    k = cases.dit_case("dit_hs64")
+    cfg = k["cfg"]
+    den = M.Denoiser(dev_params(k["params"]), cfg, "bf16")
+    args = [dev(k["pooled"]), dev(k["captions"]), dev(k["latent"]), dev(k["timesteps"])]
+    args2 = [a.clone() for a in args]
+    args2[2] = args2[2] * 0.5 + 0.25
+    want1, want2 = den(*args).clone(), den(*args2).clone()
+    torch.cuda.synchronize()
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    outs = []
+    for i in range(6):  # nothing synchronises the host between these calls
+        with torch.cuda.stream(s1 if i % 2 == 0 else s2):
+            outs.append(den(*(args if i % 2 == 0 else args2), out=torch.empty_like(args[2])))
+    torch.cuda.synchronize()
+    for i, o in enumerate(outs):
+        assert torch.equal(o, want1 if i % 2 == 0 else want2)
+    den.ctx.close()
+
+
 def test_cfg_euler_step_equals_forward_then_formula():
     """The guided Euler step writes latent + dsigma * (v_u + g * (v_c - v_u)) from the same velocities the plain forward
     returns (closed form; the reference has no sampler), for an odd grid so that pixels outside the patch grid are covered."""
