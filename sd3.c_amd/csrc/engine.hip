@@ -833,8 +833,13 @@ int sd3_ctx_set_stream(sd3_ctx* ctx, void* stream) {
     DeviceGuard g(ctx->device);
     if (!g.ok) return fail(SD3_ERR_HIP, "cannot select device %d", ctx->device);
     if (!ctx->order_event) SD3_HIP_TRY(hipEventCreateWithFlags(&ctx->order_event, hipEventDisableTiming));
-    SD3_HIP_TRY(hipEventRecord(ctx->order_event, ctx->stream));
-    SD3_HIP_TRY(hipStreamWaitEvent(ST(stream), ctx->order_event, 0));
+    if (hipEventRecord(ctx->order_event, ctx->stream) == hipSuccess) {
+        SD3_HIP_TRY(hipStreamWaitEvent(ST(stream), ctx->order_event, 0));
+    } else {
+        // the old stream no longer exists (its owner destroyed it): whatever ran on it is ordered by a device-wide wait instead
+        (void)hipGetLastError();
+        SD3_HIP_TRY(hipDeviceSynchronize());
+    }
     ctx->stream = ST(stream);
     return SD3_OK;
 }
