@@ -71,6 +71,11 @@ __device__ __forceinline__ float gelu_tanh_precise(float x) {
 }
 __device__ __forceinline__ float silu_precise(float x) { return x / (1.0f + expf(-x)); }
 
+// the value of another lane of the same row of 16 lanes, chosen by a DPP control word (no trip through the LDS crossbar)
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, false));
+}
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);

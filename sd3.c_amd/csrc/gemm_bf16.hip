@@ -461,11 +461,16 @@ __device__ __forceinline__ void gemm_tile(const Prob& pr, const int wg, char* sm
                         // explicit fused multiply-adds: left to the compiler, each unrolled copy of this code may pick a different
                         // product to fuse, and a row's result would depend on where in the tile it sits
                         float ss = fmaf(v[3], v[3], fmaf(v[2], v[2], fmaf(v[1], v[1], v[0] * v[0])));
-                        ss += __shfl_xor(ss, 1, 64);
-                        ss += __shfl_xor(ss, 2, 64);
-                        ss += __shfl_xor(ss, 4, 64);
-                        ss += __shfl_xor(ss, 8, 64);
-                        const float inv = 1.0f / sqrtf(1e-6f + ss * (1.0f / 64.0f));
+                        // butterfly over the 16 lanes with data-parallel-primitive moves (no trip through the LDS crossbar): lanes ^1 and ^2
+                        // by quad permutes; after those every quad holds one value, so mirroring the half row (i <-> 7-i) and then the
+                        // row (i <-> 15-i) pairs the same partial sums as lanes ^4 and ^8 would
+                        ss += dpp_move<0xB1>(ss);   // quad_perm [1,0,3,2]
+                        ss += dpp_move<0x4E>(ss);   // quad_perm [2,3,0,1]
+                        ss += dpp_move<0x141>(ss);  // row_half_mirror
+                        ss += dpp_move<0x140>(ss);  // row_mirror
+                        // (the hardware's reciprocal square root, 1 ulp: a divide and a square root here cost 0.2 ms per forward,
+                        // and the result is rounded to bf16 anyway)
+                        const float inv = __builtin_amdgcn_rsqf(1e-6f + ss * (1.0f / 64.0f));
                         const float4 w4 = *reinterpret_cast<const float4*>((third == 0 ? epi.gate : epi.resid) + (n0 & 63));
                         v[0] = (v[0] * inv) * w4.x; v[1] = (v[1] * inv) * w4.y; v[2] = (v[2] * inv) * w4.z; v[3] = (v[3] * inv) * w4.w;
                     }
