@@ -57,8 +57,10 @@ __global__ void __launch_bounds__(256) small_linear_kernel(const float* __restri
 #pragma unroll
         for (int j = 0; j < 4; j++) acc[m][j] = 0.f;
 
+    constexpr int UNROLL_K = M <= 2 ? 8 : 4;
     if (c0 < job.N) {
-#pragma unroll 8  // eight weight rows in flight per thread (measured: 4 and 16 are slower)
+        // weight rows in flight per thread: eight with one or two rows of x (measured: 4 and 16 are slower), four with more rows (registers)
+#pragma unroll UNROLL_K
         for (int k = kbeg; k < kend; k++) {
             float w[4];
             if (VEC) {
