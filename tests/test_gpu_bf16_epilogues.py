@@ -183,6 +183,51 @@ def test_grouping_plans_at_block_shapes_give_identical_bits_and_match_float64():
     assert rel_l2(host(base["big"][rows]), host(ref)) <= 4e-3
 
 
+@pytest.mark.parametrize("epi", [1, 5])
+def test_row_split_over_two_launches_gives_identical_bits(epi):
+    """A many-row problem whose 256x256 tiles leave a partial round (here 8000 x 4608: 576 tiles on 256 compute units) runs its first
+    rows as full rounds of 256x256 tiles and the rest, with the few-row problem, as 128x128 tiles in a second launch. Same bits as
+    without the split and as either tile shape alone, and a float64 check of rows on both sides of the split."""
+    g = torch.Generator(device="cuda").manual_seed(54 + epi)
+    K, N = 128, 4608
+    big_A = torch.randn((8000, K), device="cuda", generator=g).bfloat16()
+    small_A = torch.randn((300, K), device="cuda", generator=g).bfloat16()
+    Wp = [(0.1 * torch.randn((N, K), device="cuda", generator=g)).bfloat16() for _ in range(2)]
+    bias = [0.1 * torch.randn(N, device="cuda", generator=g) for _ in range(2)]
+    rq, rk = (1 + 0.1 * torch.randn(64, device="cuda", generator=g) for _ in range(2))
+
+    def run(tile, split):
+        outs = [torch.zeros((a.shape[0], N), device="cuda", dtype=torch.bfloat16) for a in (big_A, small_A)]
+        ps = []
+        for a, w, b, o in zip((big_A, small_A), Wp, bias, outs):
+            p = L.GemmBf16Problem(A=a.data_ptr(), wpacked=w.data_ptr(), bias=b.data_ptr(), out=o.data_ptr(), M=a.shape[0], N=N, K=K)
+            if epi == 5:
+                p.rms_q, p.rms_k = rq.data_ptr(), rk.data_ptr()
+            ps.append(p)
+        try:
+            L.call("sd3_tune", b"gemm_bf16_tile", tile)
+            L.call("sd3_tune", b"gemm_bf16_row_split", split)
+            launch(ps, epi, False)
+        finally:
+            L.call("sd3_tune", b"gemm_bf16_tile", 0)
+            L.call("sd3_tune", b"gemm_bf16_row_split", 1)
+        return outs
+
+    base = run(0, 1)  # the split plan (the default choice at this shape)
+    for tile, split in ((0, 0), (256, 1), (128, 1)):
+        other = run(tile, split)
+        assert torch.equal(other[0], base[0]) and torch.equal(other[1], base[1]), (tile, split)
+    rows = torch.tensor([0, 255, 7167, 7168, 7169, 7999], device="cuda")  # the split falls between rows 7167 and 7168
+    ref = big_A[rows].double() @ Wp[0].double().t() + bias[0].double()
+    if epi == 1:
+        ref = torch.nn.functional.gelu(ref, approximate="tanh")
+    else:
+        q, k, v = ref.view(len(rows), 3, N // 192, 64).unbind(1)
+        nrm = lambda t, w: t * torch.rsqrt(t.pow(2).mean(-1, keepdim=True) + 1e-6) * w.double()  # noqa: E731
+        ref = torch.stack([nrm(q, rq), nrm(k, rk), v], 1).reshape(len(rows), N)
+    assert rel_l2(host(base[0][rows]), host(ref)) <= 4e-3
+
+
 def test_grouped_gemm_argument_errors():
     none = C.c_void_p(0)
     p = L.GemmBf16Problem(M=4, N=192, K=64)
