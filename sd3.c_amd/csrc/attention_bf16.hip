@@ -574,8 +574,11 @@ int g_attention_context_splits = -1;  // -1: chosen from the sizes; 0: never spl
 int attention_bf16_context_splits(int Tc, int Tx) {
     const int nt_all = (Tc + Tx + BKV - 1) / BKV;
     if (Tc <= 0 || Tc > BQ || Tx < 4 * BQ || nt_all < 16 || g_attention_context_splits == 0) return 0;
-    const int want = g_attention_context_splits > 0 ? g_attention_context_splits : 4;
-    return want < 2 ? 2 : (want > 8 ? 8 : want);
+    int S = g_attention_context_splits > 0 ? g_attention_context_splits : 4;
+    S = S < 2 ? 2 : (S > 8 ? 8 : S);
+    // every split must own at least one key tile: with ceil(nt_all / S) tiles each, the last one starts at (S-1) * that
+    while (S > 1 && ((nt_all + S - 1) / S) * (S - 1) >= nt_all) S--;
+    return S > 1 ? S : 0;
 }
 size_t attention_bf16_split_workspace_floats(int B, int NH, int Tc, int splits) {
     const size_t items = (size_t)B * NH * ((Tc + BQ - 1) / BQ) * splits;

@@ -176,6 +176,26 @@ def test_block_bf16_vs_fp32(dual, discard, Tc, Tx):
         assert rel_l2(c16, c32) <= BF16_REL_L2
 
 
+@pytest.mark.parametrize("splits", [0, 3, 8, -1])
+def test_block_bf16_with_every_context_split_setting(splits):
+    """The attention of a block with many latent and few context tokens is taken apart by queries, the context queries split along
+    the keys (17 key tiles here, which 8 splits cannot share without leaving one empty: the library then uses fewer). Whatever the
+    setting, the block stays within the bf16 criterion of the fp32 path, and the latent rows do not depend on it at all."""
+    from sd3_c_amd import lib as L_
+    k = _wide_case(1, 20, 1040, True, False, 61, C=128, NH=2)
+    c32, x32 = run_gpu_block(k, "fp32")
+    try:
+        L_.call("sd3_tune", b"attention_context_splits", splits)
+        c16, x16 = run_gpu_block(k, "bf16")
+        L_.call("sd3_tune", b"attention_context_splits", 0)
+        c0, x0 = run_gpu_block(k, "bf16")
+    finally:
+        L_.call("sd3_tune", b"attention_context_splits", -1)
+    assert rel_l2(x16, x32) <= BF16_REL_L2 and rel_l2(c16, c32) <= BF16_REL_L2
+    assert np.array_equal(x16, x0)                 # latent rows: same kernel path, same bits
+    assert rel_l2(c16, c0) <= 2e-3                 # context rows: merged partial sums, bf16 rounding apart
+
+
 def test_block_missing_weight_and_bad_shapes():
     from sd3_c_amd import lib as L_
     k = cases.block_case("block_dual_hs64")
