@@ -75,7 +75,13 @@ __global__ void __launch_bounds__(256) ln_mod_vec_kernel(const LnSegPair<OutT> s
         }
     }
     const float rstd = 1.0f / sqrtf(wave_sum(q) / C + eps);
-    const long long b = row / T;
+    long long b = 0;  // batch element of the row: with at most 8 of them a few comparisons instead of a 64-bit division
+    if (g.rows <= 8LL * T) {
+#pragma unroll
+        for (int k = 1; k < 8; k++) b += (row >= (long long)k * T) ? 1 : 0;
+    } else {
+        b = row / T;
+    }
     const float4* sh = g.shift ? reinterpret_cast<const float4*>(g.shift + b * mod_ld) : nullptr;
     const float4* sc = g.scale ? reinterpret_cast<const float4*>(g.scale + b * mod_ld) : nullptr;
     const float4* sh2 = g.shift2 ? reinterpret_cast<const float4*>(g.shift2 + b * mod_ld) : nullptr;

@@ -40,10 +40,9 @@ __global__ void __launch_bounds__(256) small_linear_kernel(const float* __restri
     const int col_base = blockIdx.x * 128;
     if (col_base >= job.N) return;
     const int tid = threadIdx.x;
-    for (int idx = tid; idx < M * K; idx += 256) {
-        const int m = idx / K, k = idx - m * K;
-        smem[k * M + m] = (m < m_real) ? x[(long long)m * K + k] : 0.f;
-    }
+#pragma unroll
+    for (int m = 0; m < M; m++)
+        for (int k = tid; k < K; k += 256) smem[k * M + m] = (m < m_real) ? x[(long long)m * K + k] : 0.f;
     __syncthreads();
 
     const int cl = tid & 31, ks = tid >> 5;
