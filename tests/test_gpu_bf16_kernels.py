@@ -92,6 +92,37 @@ def test_flash_attention_bf16_taken_apart_by_queries_with_key_splits(B, T0, T1, 
         L.call("sd3_flash_attention_bf16_split", qkv0.data_ptr(), qkv1.data_ptr(), out0.data_ptr(), out1.data_ptr(), B, T0, T1, NH, HS, S, ws.data_ptr(), 16, None)
 
 
+def test_flash_attention_bf16_headline_size_properties():
+    """Size-independent properties at the benchmark's attention shape (B=2, 24 heads of 64, 154 text + 4096 image tokens), where no
+    CPU reference finishes: (1) with V = 1 every output is 1 (each row of the softmax sums to one, whatever the scores);
+    (2) permuting the image tokens' keys and values together leaves every output unchanged up to the order of summation."""
+    B, T0, T1, NH, HS = 2, 154, 4096, 24, 64
+    C = NH * HS
+    g = torch.Generator(device="cuda").manual_seed(99)
+    qkv0 = torch.randn((B * T0, 3 * C), device="cuda", generator=g).bfloat16()
+    qkv1 = torch.randn((B * T1, 3 * C), device="cuda", generator=g).bfloat16()
+
+    def run(a0, a1):
+        o0 = torch.zeros((B * T0, C), device="cuda", dtype=torch.bfloat16)
+        o1 = torch.zeros((B * T1, C), device="cuda", dtype=torch.bfloat16)
+        L.call("sd3_flash_attention_bf16", a0.data_ptr(), a1.data_ptr(), o0.data_ptr(), o1.data_ptr(), None, None, None, None, B, T0, T1, NH, HS, None)
+        torch.cuda.synchronize()
+        return o0.float(), o1.float()
+
+    ones0, ones1 = qkv0.clone(), qkv1.clone()
+    ones0[:, 2 * C:] = 1
+    ones1[:, 2 * C:] = 1
+    o0, o1 = run(ones0, ones1)
+    assert float((o0 - 1).abs().max()) <= 1e-2 and float((o1 - 1).abs().max()) <= 1e-2
+    base0, base1 = run(qkv0, qkv1)
+    perm = torch.randperm(T1, device="cuda", generator=g)
+    shuffled = qkv1.view(B, T1, 3, C).clone()
+    shuffled[:, :, 1:] = shuffled[:, perm][:, :, 1:]     # keys and values move together, queries stay where they are
+    p0, p1 = run(qkv0, shuffled.view(B * T1, 3 * C).contiguous())
+    assert float((p0 - base0).abs().max()) <= 0.02 and float((p1 - base1).abs().max()) <= 0.02
+    assert rel_l2(host(p1), host(base1)) <= 5e-3 and rel_l2(host(p0), host(base0)) <= 5e-3
+
+
 def test_flash_attention_bf16_without_qk_norm_and_ones_v():
     B, T0, T1, NH, HS = 1, 10, 200, 2, 64
     C = NH * HS
