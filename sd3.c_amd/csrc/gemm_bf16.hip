@@ -46,7 +46,7 @@ __device__ __forceinline__ void wait_vmcnt() {
 // bands of GROUP_M tile rows, so that the ~32 tiles an XCD works on at a time share a few A row panels and W column
 // panels inside that L2 instead of each pulling its own panels from the fabric.
 __device__ __forceinline__ void tile_of_workgroup(int wg, int tiles_m, int tiles_n, int& tile_m, int& tile_n) {
-    constexpr int XCDS = 8, GROUP_M = 4;
+    constexpr int XCDS = 8, GROUP_M = 2;  // measured over 1, 2, 3, 4, 8, 16 on the 24-block forward: 2 is the fastest
     const int total = tiles_m * tiles_n;
     const int xcd = wg % XCDS, local = wg / XCDS;
     const int per = (total + XCDS - 1) / XCDS, tall = (total % XCDS) ? (total % XCDS) : XCDS;  // `tall` XCDs get `per` tiles, the rest per-1
@@ -201,7 +201,8 @@ __device__ __forceinline__ void gemm_tile(const Prob& pr, const int wg, char* sm
         // A fragments: one buffer (the fragment of the next step replaces a[i] as soon as row block i is done), except for the last
         // TAIL row blocks, which have two so that no fragment read is left to issue behind the last matrix instructions of a step
         // (it would be waited for at once); B fragments: two buffers
-        constexpr int TAIL = MI >= 6 ? 3 : MI / 2, HEAD = MI - TAIL;
+        // (one such row block for the large tiles: more of them cost registers, which the gated fp32 epilogue then spills)
+        constexpr int TAIL = MI >= 6 ? 1 : MI / 2, HEAD = MI - TAIL;
         static_assert(HEAD >= TAIL && TAIL >= 1, "every tail fragment is fetched behind a head row block");
         bf16x8_t a[HEAD], at[2][TAIL], b[2][NJ];
         auto a_addr = [&](const char* st, int s, int i) { return reinterpret_cast<const bf16x8_t*>(st + a_off + i * 16 * 128 + (((4 * s + lg) ^ sw) * 16)); };
