@@ -15,6 +15,8 @@
 // instructions; a workgroup of 4 wavefronts shares each 64-key tile. K tiles go global -> LDS directly
 // (global_load_lds_dwordx4) into 128-byte rows with XOR-swizzled 16-byte chunks; tiles are double-buffered with one
 // barrier per tile.
+#include <type_traits>
+
 #include "common.hpp"
 
 namespace sd3 {
@@ -166,21 +168,15 @@ __global__ void __launch_bounds__(NW * 64, 2) flash_attn_bf16_kernel(const AttnS
     }
 
     f32x16_t oacc[2][2];  // [d block][query block]
-#pragma unroll
-    for (int i = 0; i < 2; i++)
-#pragma unroll
-        for (int j = 0; j < 2; j++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) oacc[i][j][r] = 0.f;
     // Softmax reference point m_run per query (any value works as long as numerator and denominator use the same one) and
     // this lane's share l_run of the row sum. The matrix unit subtracts the reference and masks keys beyond the sequence:
     // a score block starts from AUX . NEGM, where AUX[key][k=0] = 1, AUX[key][k=1] = (key beyond the sequence),
     // NEGM[k=0][query] = -m_run (kept representable in bf16), NEGM[k=1][query] = -1e30 and everything else is zero.
-    float m_run[2] = {0.f, 0.f}, l_run[2] = {0.f, 0.f};
+    // While the reference is zero and no key of a block is masked that product is zero, and the loop over such tiles
+    // ("fast" tiles below) leaves it out.
+    float m_run[2], l_run[2];
     const uint32_t NEG_BIG_HI = pack_bf16x2(0.f, -1e30f);  // bf16(-1e30) in the upper half
     Frag negm_f[2];
-#pragma unroll
-    for (int qb = 0; qb < 2; qb++) negm_f[qb].u = make_uint4(lk == 0 ? NEG_BIG_HI : 0u, 0u, 0u, 0u);
     // a partial row sum of 16 probabilities above this bound (or infinite) moves the reference
     constexpr float L_BOUND = 1073741824.0f;  // 2^30
 
@@ -282,22 +278,50 @@ __global__ void __launch_bounds__(NW * 64, 2) flash_attn_bf16_kernel(const AttnS
     Frag pf[2][2];      // pf[qb][j]: its probabilities as P^T operands
     bf16x8_t kf[4];     // K fragments of the key half whose scores are being issued
     uint2 vfr[8];       // V^T fragments of the key half whose PV products are being issued: [j][d block][keys 0-3 | 8-11 of the step]
-#pragma unroll
-    for (int i = 0; i < 8; i++) vfr[i] = make_uint2(0u, 0u);
-#pragma unroll
-    for (int qb = 0; qb < 2; qb++)
-#pragma unroll
-        for (int j = 0; j < 2; j++) pf[qb][j].u = make_uint4(0u, 0u, 0u, 0u);
-
     // AUX rows for keys key_base + l32: one persistent operand whose first register alone changes from unit to unit
     Frag aux;
-    aux.u = make_uint4(0u, 0u, 0u, 0u);
-    const int first_masked = T - l32;  // key_base >= first_masked  <=>  key key_base + l32 lies beyond the sequence
-    auto scores = [&](int qb, int key_base) {
-        aux.u.x = (key_base >= first_masked) ? 0x3f803f80u : 0x00003f80u;
-        sacc[qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(aux.v, negm_f[qb].v, zero, 0, 0, 0);
+    int first_masked;  // key_base >= first_masked  <=>  key key_base + l32 lies beyond the sequence
+    auto reset = [&]() {  // the state in front of an item's first tile
 #pragma unroll
-        for (int ks = 0; ks < 4; ks++) sacc[qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[ks], qf[qb][ks].v, sacc[qb], 0, 0, 0);
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) oacc[i][j][r] = 0.f;
+#pragma unroll
+        for (int qb = 0; qb < 2; qb++) {
+            l_run[qb] = 0.f;
+#pragma unroll
+            for (int j = 0; j < 2; j++) pf[qb][j].u = make_uint4(0u, 0u, 0u, 0u);
+        }
+#pragma unroll
+        for (int i = 0; i < 8; i++) vfr[i] = make_uint2(0u, 0u);
+    };
+    // The operands of the general path that say "reference zero". Called in front of an item's first tile and again behind the fast
+    // tiles, which use none of this: built from a value the optimiser cannot trace, so that the second call does not simply keep
+    // the results of the first in registers across the fast tiles, where registers are what the instruction schedule is short of.
+    auto zero_reference = [&]() {
+        int lane_o = (int)__lane_id();
+        asm volatile("" : "+v"(lane_o));
+        first_masked = T - (lane_o & 31);
+#pragma unroll
+        for (int qb = 0; qb < 2; qb++) {
+            m_run[qb] = 0.f;
+            negm_f[qb].u = make_uint4((lane_o >> 5) == 0 ? NEG_BIG_HI : 0u, 0u, 0u, 0u);
+        }
+        aux.u = make_uint4(0u, 0u, 0u, 0u);
+    };
+    auto scores = [&](auto fast, int qb, int key_base) {
+        constexpr bool FAST = decltype(fast)::value;
+        if (FAST) {
+            sacc[qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[0], qf[qb][0].v, zero, 0, 0, 0);
+        } else {
+            aux.u.x = (key_base >= first_masked) ? 0x3f803f80u : 0x00003f80u;
+            sacc[qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(aux.v, negm_f[qb].v, zero, 0, 0, 0);
+            sacc[qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[0], qf[qb][0].v, sacc[qb], 0, 0, 0);
+        }
+#pragma unroll
+        for (int ks = 1; ks < 4; ks++) sacc[qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[ks], qf[qb][ks].v, sacc[qb], 0, 0, 0);
     };
     auto load_k = [&](int stage_byte, int kb) {
 #pragma unroll
@@ -355,10 +379,13 @@ __global__ void __launch_bounds__(NW * 64, 2) flash_attn_bf16_kernel(const AttnS
 #pragma unroll
             for (int r = 2; r < 16; r += 2) tmax = fmaxf(tmax, fmaxf(sacc[qb][r], sacc[qb][r + 1]));
             // lanes l and l^32 hold the two key halves of the same query and feed the same accumulators: same reference
-            const float m_new = fmaxf(m_old, m_old + fmaxf(tmax, __shfl_xor(tmax, 32, 64)));
+            // (forced = the first unit of a query block: nothing has been accumulated, the reference is still zero and goes to that unit's
+            // maximum wherever that lies, also far below zero, where a reference of zero would turn every probability into nothing)
+            const float pair_max = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+            const float m_new = force ? pair_max : fmaxf(m_old, m_old + pair_max);
             const uint32_t negm_bits = pack_bf16x2(-m_new, 0.f) & 0xffffu;
             const float m_ref = -__uint_as_float(negm_bits << 16);
-            const float alpha = __builtin_amdgcn_exp2f(m_old - m_ref);
+            const float alpha = force ? 1.0f : __builtin_amdgcn_exp2f(m_old - m_ref);
             m_run[qb] = m_ref;
             negm_f[qb].u.x = lk == 0 ? (negm_bits | NEG_BIG_HI) : 0u;
             l_run[qb] *= alpha;
@@ -373,53 +400,51 @@ __global__ void __launch_bounds__(NW * 64, 2) flash_attn_bf16_kernel(const AttnS
         }
         l_run[qb] += inc;
     };
-    // one matrix instruction, then a few vector instructions, nine times: the mix of one pipeline step
-    auto interleave = [&]() {
+    // one matrix instruction, then a few vector instructions, nine times: the mix of one pipeline step of the general path.
+    // (Fast tiles go without: every such pattern tried there -- 1:2 to 1:5, pairs, with the transcendental class named -- measured
+    // 7 % slower than what the compiler's own scheduler does with the shorter step.)
+    auto interleave = [&](auto fast) {
+        if (decltype(fast)::value) return;
 #pragma unroll
         for (int i = 0; i < 9; i++) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
             __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
         }
     };
+    // A fast tile keeps the reference at zero and only adds up; whether that was safe is looked at once per tile (verdict below).
+    auto account = [&](auto fast, int qb, float inc, bool force) {
+        if (decltype(fast)::value) {
+            l_run[qb] += inc;
+        } else {
+            settle(qb, inc, force);
+        }
+    };
 
-    // prologue: tiles 0 and 1 on their way, tile 0 visible, scores of the first unit issued
-    advance(kv0);
-    fetch_tile(0);
-    if (NORM) store_k_normed(kv0, 0);
-    if (nt > 1) {
-        advance(kv0 + BKV);
-        fetch_tile(STAGE_BYTES);
-        __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8) | 4);  // vmcnt(4): all but the four loads of tile 1
-    } else {
-        __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8));
-    }
-    __syncthreads();
-    load_k(0, 0);
-    scores(0, kv0);
-    int st_cur = 0, st_nxt = STAGE_BYTES, st_ld = 2 * STAGE_BYTES;  // stages of tiles t, t+1, t+2
-
-    for (int t = 0; t < nt; t++) {
+    // Stages of tiles t, t+1, t+2
+    int st_cur, st_nxt, st_ld;
+    // One tile of the pipeline: four steps. FAST tiles are those in which no key is masked and the reference is known to be zero.
+    auto tile = [&](auto fast, int t) {
         float inc;
         // ---- step (t, 0, 0): PV of (t-1,1,1), each half followed by the fetch of V of key half 0 into the registers it
         //      frees; scores of (t,0,1); then fetch K of half 1 ----
         pv(1, 0);
         load_v(st_cur, 0, 0);
-        scores(1, kv0 + t * BKV);
+        scores(fast, 1, kv0 + t * BKV);
         load_k(st_cur, 1);
         inc = probs(0);
         pv(1, 1);
         load_v(st_cur, 0, 1);
-        interleave();
-        settle(0, inc, t == 0);
+        interleave(fast);
+        account(fast, 0, inc, t == 0);
         // ---- step (t, 0, 1): PV of (t,0,0); scores of (t,1,0) ----
         lds_wait_first4(vfr);
         pv(0, 0);
-        scores(0, kv0 + t * BKV + 32);
+        scores(fast, 0, kv0 + t * BKV + 32);
         inc = probs(1);
         lds_wait_last4(vfr);
         pv(0, 1);
-        interleave();
-        settle(1, inc, t == 0);
+        interleave(fast);
+        account(fast, 1, inc, t == 0);
         // ---- step (t, 1, 0): tile t+1 becomes visible and the loads of tile t+2 set off (past the end: the last tile once
         //      more, into a stage nobody reads again); PV of (t,0,1) and fetch of V of key half 1; scores of (t,1,1); then
         //      fetch K of half 0 of tile t+1 (past the last tile: stale LDS, feeding scores that are never used) ----
@@ -430,43 +455,109 @@ __global__ void __launch_bounds__(NW * 64, 2) flash_attn_bf16_kernel(const AttnS
         fetch_tile(st_ld);
         pv(1, 0);
         load_v(st_cur, 1, 0);
-        scores(1, kv0 + t * BKV + 32);
+        scores(fast, 1, kv0 + t * BKV + 32);
         load_k(st_nxt, 0);
         inc = probs(0);
         pv(1, 1);
         load_v(st_cur, 1, 1);
-        interleave();
-        settle(0, inc, false);
+        interleave(fast);
+        account(fast, 0, inc, false);
         // ---- step (t, 1, 1): PV of (t,1,0); scores of (t+1,0,0) ----
         lds_wait_first4(vfr);
         pv(0, 0);
-        scores(0, kv0 + t * BKV + BKV);
+        scores(fast, 0, kv0 + t * BKV + BKV);
         inc = probs(1);
         lds_wait_last4(vfr);
         pv(0, 1);
-        interleave();
-        settle(1, inc, false);
+        interleave(fast);
+        account(fast, 1, inc, false);
         const int tmp = st_cur;
         st_cur = st_nxt;
         st_nxt = st_ld;
         st_ld = tmp;
+    };
+
+    // Fast tiles: the leading tiles whose units, and the unit whose scores the last of them issues (the first of the next tile), lie
+    // wholly inside the sequence. With the reference at zero a probability is 2^score, which is as good as any other reference while
+    // the row sums stay inside the range of fp32: every lane's partial row sum must have left the denormal range (a row whose scores
+    // are all hugely negative would otherwise be lost) and stay below 2^40 (far from overflow; a row sum of 4250 normalised head
+    // vectors with unit weights is below 2^24). Row sums only grow and an infinity stays one, so one look behind the last fast
+    // tile is enough (looking inside the loop as well was tried: the extra control flow makes the register allocator spill
+    // hundreds of registers). A lane that sees otherwise raises a flag in LDS, a barrier follows, every wavefront reads the
+    // flag, and the whole item starts again with every tile going through the general path. Nothing has been written by then,
+    // so values that overflowed in the meantime are simply dropped; an input like that pays for the fast tiles in vain.
+    __shared__ int unsafe_flag;
+    constexpr float L_TINY = 5.421010862427522e-20f /* 2^-64 */, L_HUGE = 1099511627776.0f /* 2^40 */;
+    int n_fast = (kv0 + nt * BKV <= T) ? nt : min(nt, (T - kv0 - 32) / BKV);
+    if (NORM || n_fast < 4) n_fast = 0;
+    const std::integral_constant<bool, true> FAST_TILE;
+    const std::integral_constant<bool, false> ANY_TILE;
+
+    for (;;) {
+        reset();
+        zero_reference();
+        if (tid == 0) unsafe_flag = 0;
+        // prologue: tiles 0 and 1 on their way, tile 0 visible, scores of the first unit issued
+        // (the first key is hidden from the optimiser here: otherwise the address arithmetic of the prologue, which does not
+        // change from one attempt to the next, is moved in front of this loop and its results are kept in scratch memory)
+        int first_key = kv0;
+        asm volatile("" : "+s"(first_key));
+        advance(first_key);
+        fetch_tile(0);
+        if (NORM) store_k_normed(kv0, 0);
+        if (nt > 1) {
+            advance(first_key + BKV);
+            fetch_tile(STAGE_BYTES);
+            __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8) | 4);  // vmcnt(4): all but the four loads of tile 1
+        } else {
+            __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8));
+        }
+        __syncthreads();
+        load_k(0, 0);
+        scores(ANY_TILE, 0, kv0);
+        st_cur = 0, st_nxt = STAGE_BYTES, st_ld = 2 * STAGE_BYTES;
+
+        // verdict on the fast tiles so far, the same for every wavefront of the workgroup: flags raised in front of a barrier, read behind it
+        auto unsafe = [&]() -> bool {
+            const bool bad = !(l_run[0] <= L_HUGE && l_run[1] <= L_HUGE) || l_run[0] < L_TINY || l_run[1] < L_TINY;
+            volatile int* flag = &unsafe_flag;
+            if (__any(bad)) *flag = 1;
+            __syncthreads();
+            return __builtin_amdgcn_readfirstlane(*flag) != 0;
+        };
+        for (int t = 0; t < n_fast; t++) tile(FAST_TILE, t);
+        const bool redo = n_fast > 0 && unsafe();
+        if (!redo) {
+            if (n_fast > 0) zero_reference();
+            for (int t = n_fast; t < nt; t++) tile(ANY_TILE, t);
+            break;
+        }
+        // start again without fast tiles, once every wavefront is done with the LDS stages and no load into them is in flight
+        __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8));
+        __syncthreads();
+        n_fast = 0;
     }
     pv(1, 0);  // PV of the last unit
     pv(1, 1);
     __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8));  // the redundant loads issued past the last tile have landed before LDS is reused
 
+    // The lane's coordinates once more, derived behind the loops from a value the optimiser cannot trace back: index arithmetic for
+    // the stores below would otherwise be computed up front and carried, through scratch memory, across the loops.
+    int lane_e = (int)__lane_id();
+    asm volatile("" : "+v"(lane_e));
+    const int l32e = lane_e & 31, lke = lane_e >> 5;
     // ---- an item of a split: leave the unnormalised accumulators, the reference and the row sum for the combining kernel ----
     if (s.kv_splits > 1) {
 #pragma unroll
         for (int qb = 0; qb < 2; qb++) {
-            const long long prow = (long long)item * BQ + wave * QW + qb * 32 + l32;
+            const long long prow = (long long)item * BQ + wave * QW + qb * 32 + l32e;
             const float l_tot = l_run[qb] + __shfl_xor(l_run[qb], 32, 64);
-            if (lk == 0) *reinterpret_cast<float2*>(s.part_ml + prow * 2) = make_float2(m_run[qb], l_tot);
+            if (lke == 0) *reinterpret_cast<float2*>(s.part_ml + prow * 2) = make_float2(m_run[qb], l_tot);
 #pragma unroll
             for (int db = 0; db < 2; db++)
 #pragma unroll
                 for (int g = 0; g < 4; g++)
-                    *reinterpret_cast<float4*>(s.part_o + prow * HS + db * 32 + 8 * g + 4 * lk) =
+                    *reinterpret_cast<float4*>(s.part_o + prow * HS + db * 32 + 8 * g + 4 * lke) =
                         make_float4(oacc[db][qb][4 * g + 0], oacc[db][qb][4 * g + 1], oacc[db][qb][4 * g + 2], oacc[db][qb][4 * g + 3]);
         }
         return;
@@ -482,19 +573,19 @@ __global__ void __launch_bounds__(NW * 64, 2) flash_attn_bf16_kernel(const AttnS
         for (int db = 0; db < 2; db++)
 #pragma unroll
             for (int g = 0; g < 4; g++) {
-                const int d0 = db * 32 + 8 * g + 4 * lk;
+                const int d0 = db * 32 + 8 * g + 4 * lke;
                 const uint2 v = make_uint2(pack_bf16x2(oacc[db][qb][4 * g + 0] * inv, oacc[db][qb][4 * g + 1] * inv),
                                            pack_bf16x2(oacc[db][qb][4 * g + 2] * inv, oacc[db][qb][4 * g + 3] * inv));
-                *reinterpret_cast<uint2*>(&Ow[(qb * 32 + l32) * O_PITCH + d0]) = v;
+                *reinterpret_cast<uint2*>(&Ow[(qb * 32 + l32e) * O_PITCH + d0]) = v;
             }
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    // 64 rows x 8 chunks per wavefront = 512 chunks, 8 per lane
+    // 64 rows x 8 chunks per wavefront = 512 chunks, 8 per lane_e
 #pragma unroll
     for (int i = 0; i < 8; i++) {
-        const int c = lane + i * 64;
+        const int c = lane_e + i * 64;
         const int row = c >> 3, ch = c & 7;
         const int t = q0 + row;
         if (t < TQ) {

@@ -197,6 +197,53 @@ def test_flash_attention_bf16_late_maximum_moves_the_reference():
     assert float((out.float() - ref).abs().max()) <= 0.05
 
 
+@pytest.mark.parametrize("case", ["overflow_mid", "overflow_to_inf", "first_tile_vanishes", "everything_vanishes", "harmless"])
+def test_flash_attention_bf16_fast_tiles_give_way_to_the_general_path(case):
+    """Tiles in which no key is masked run with the softmax reference fixed at zero, as long as every lane's row sums stay between
+    2^-64 (after the first tile) and 2^40; otherwise the work item starts again on the general path. Cases: scores of 2^40 and more
+    in the middle of the sequence; scores beyond the fp32 exponent range (the fast tiles produce infinities before the check
+    sees them); queries whose scores against the whole first tile are below -100 (their probabilities there round to nothing)
+    while later keys are ordinary; queries whose scores against every key are below -100 (with a reference of zero their row sums
+    would be zero); and an ordinary input, which stays on the fast tiles. Reference as in the test above."""
+    B, T1, NH, HS = 1, 1000, 2, 64
+    C = NH * HS
+    g = torch.Generator(device="cuda").manual_seed(23)
+    qkv = torch.randn((B * T1, 3 * C), device="cuda", generator=g)
+    if case == "overflow_mid":
+        qkv[400:405, C:2 * C] *= 12.0
+    elif case == "overflow_to_inf":
+        qkv[130:140, C:2 * C] *= 60.0
+    elif case == "first_tile_vanishes":
+        u = torch.nn.functional.normalize(torch.randn(NH, HS, device="cuda", generator=g), dim=-1)
+        qkv[:64, C:2 * C] = (-40.0 * u).reshape(1, C) + 0.1 * qkv[:64, C:2 * C]     # the first tile's keys all point one way ...
+        qkv[500:, 0:C] = (24.0 * u).reshape(1, C) + qkv[500:, 0:C]                  # ... and half of the queries the opposite way
+    elif case == "everything_vanishes":
+        u = torch.nn.functional.normalize(torch.randn(NH, HS, device="cuda", generator=g), dim=-1)
+        qkv[:, C:2 * C] = (-40.0 * u).reshape(1, C) + qkv[:, C:2 * C]
+        qkv[500:, 0:C] = (24.0 * u).reshape(1, C) + qkv[500:, 0:C]
+    qkv = qkv.bfloat16()
+    out = torch.zeros((B * T1, C), device="cuda", dtype=torch.bfloat16)
+    L.call("sd3_flash_attention_bf16", qkv.data_ptr(), None, out.data_ptr(), None, None, None, None, None, B, T1, 0, NH, HS, None)
+    q, k, v = qkv.float().view(B, T1, 3, NH, HS).unbind(2)
+    q2 = (q * (1.4426950408889634 / 8.0)).bfloat16().float()
+    s2 = torch.einsum("bqhd,bkhd->bhqk", q2, k)
+    if case == "everything_vanishes":
+        assert float(s2[:, :, 500:].max()) < -130.0  # 2^-130 is below the smallest normal fp32 number
+    elif case == "overflow_mid":
+        assert 40.0 < float(s2.max()) < 120.0
+    elif case == "overflow_to_inf":
+        assert float(s2.max()) > 200.0
+    elif case == "first_tile_vanishes":
+        assert float(s2[:, :, 500:, :64].max()) < -100.0 and float(s2[:, :, 500:, 64:].max(-1).values.min()) > -40.0
+    else:
+        assert float(s2.abs().max()) < 30.0
+    p = torch.exp2(s2 - s2.max(-1, keepdim=True).values)
+    ref = torch.einsum("bhqk,bkhd->bqhd", p / p.sum(-1, keepdim=True), v).reshape(B * T1, C)
+    assert torch.isfinite(out.float()).all()
+    assert float((out.float() - ref).abs().max()) <= 0.05
+    assert rel_l2(host(out.float()), host(ref)) <= 1e-2
+
+
 def test_cast_rounds_to_nearest_even():
     x = torch.randn(100000, device="cuda") * 100
     x[:4] = torch.tensor([0.0, -0.0, float("inf"), 1.00390625])  # the last one is exactly halfway between two bf16 values
