@@ -411,7 +411,7 @@ __global__ void __launch_bounds__(NW * 64, 2) flash_attn_bf16_kernel(const AttnS
             __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
         }
     };
-    // A fast tile keeps the reference at zero and only adds up; whether that was safe is looked at once per tile (verdict below).
+    // A fast tile keeps the reference at zero and only adds up; whether that was safe is looked at once, behind the last of them.
     auto account = [&](auto fast, int qb, float inc, bool force) {
         if (decltype(fast)::value) {
             l_run[qb] += inc;
