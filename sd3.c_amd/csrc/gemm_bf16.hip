@@ -41,14 +41,23 @@ __device__ __forceinline__ void wait_vmcnt() {
     __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
 }
 
-// Workgroup -> output tile. The hardware hands consecutive workgroup ids to the 8 XCDs in turn, and each XCD has
-// its own L2. Workgroups that land on the same XCD are therefore given a contiguous run of tiles, and runs are walked in
-// bands of GROUP_M tile rows, so that the ~32 tiles an XCD works on at a time share a few A row panels and W column
-// panels inside that L2 instead of each pulling its own panels from the fabric.
+// Workgroup -> output tile. The hardware hands consecutive workgroup ids to the 8 XCDs in turn, and each XCD has its own L2, so
+// the workgroups that land on one XCD should share as few A row panels and W column panels as possible. When the tile grid
+// divides that way, the XCDs take a 4 x 2 arrangement of rectangular blocks of it (for 32 x 24 tiles: 8 x 12 each, 8 + 12 panels
+// through that L2 instead of 4 + 24 with contiguous runs of tile rows), walked in bands of 4 tile rows so that the 32 tiles an XCD
+// works on at a time form a 4 x 8 patch. Otherwise every XCD gets a contiguous run of tiles, walked in bands of 2 tile rows
+// (measured over 1, 2, 3, 4, 8, 16 on the 24-block forward).
 __device__ __forceinline__ void tile_of_workgroup(int wg, int tiles_m, int tiles_n, int& tile_m, int& tile_n) {
-    constexpr int XCDS = 8, GROUP_M = 2;  // measured over 1, 2, 3, 4, 8, 16 on the 24-block forward: 2 is the fastest
+    constexpr int XCDS = 8, XR = 4, XC = 2, BAND = 4, GROUP_M = 2;
     const int total = tiles_m * tiles_n;
     const int xcd = wg % XCDS, local = wg / XCDS;
+    if (tiles_m % (XR * BAND) == 0 && tiles_n % XC == 0) {
+        const int bm = tiles_m / XR, bc = tiles_n / XC;  // the XCD's block: bm x bc tiles, exactly total / 8
+        const int band = local / (BAND * bc), r = local % (BAND * bc);
+        tile_m = (xcd / XC) * bm + band * BAND + r % BAND;
+        tile_n = (xcd % XC) * bc + r / BAND;
+        return;
+    }
     const int per = (total + XCDS - 1) / XCDS, tall = (total % XCDS) ? (total % XCDS) : XCDS;  // `tall` XCDs get `per` tiles, the rest per-1
     const int t = (xcd < tall) ? xcd * per + local : tall * per + (xcd - tall) * (per - 1) + local;
     const int in_group = GROUP_M * tiles_n, group = t / in_group, first_m = group * GROUP_M;
