@@ -197,6 +197,42 @@ def test_flash_attention_bf16_late_maximum_moves_the_reference():
     assert float((out.float() - ref).abs().max()) <= 0.05
 
 
+@pytest.mark.parametrize("T0,T1", [(0, 256), (0, 257), (0, 287), (0, 288), (0, 289), (0, 319), (0, 320), (0, 321), (0, 351), (0, 352), (0, 353), (0, 383),
+                                   (5, 315), (31, 289), (32, 288), (33, 330), (64, 256), (100, 412), (154, 1024 + 37)])
+def test_flash_attention_bf16_where_fast_tiles_hand_over_to_masked_ones(T0, T1):
+    """Sequence lengths on every side of the 64-key tile and 32-key half-tile boundaries, long enough (five tiles and more) for the
+    tiles without masked keys to run with the reference fixed at zero: the last one or two tiles, which hold the keys beyond the
+    sequence, go through the general path, and the unit in flight across the hand-over must be one without masked keys."""
+    B, NH, HS = 1, 2, 64
+    C = NH * HS
+    g = torch.Generator(device="cuda").manual_seed(T0 * 1000 + T1)
+    qkv0 = torch.randn((B * max(T0, 1), 3 * C), device="cuda", generator=g).bfloat16()
+    qkv1 = torch.randn((B * T1, 3 * C), device="cuda", generator=g).bfloat16()
+    rq = [1 + 0.1 * torch.randn(HS, device="cuda", generator=g) for _ in range(2)]
+    rk = [1 + 0.1 * torch.randn(HS, device="cuda", generator=g) for _ in range(2)]
+    # normalise on the host (the kernel then takes q and k as they are: the path with fast tiles)
+    def normed(qkv, T, wq, wk):
+        q, k, v = qkv.float().view(B, T, 3, NH, HS).unbind(2)
+        rms = lambda a, w: a * torch.rsqrt(a.pow(2).mean(-1, keepdim=True) + 1e-6) * w
+        return torch.stack([rms(q, wq), rms(k, wk), v], 2).reshape(B * T, 3 * C).bfloat16()
+    n0 = normed(qkv0, max(T0, 1), rq[0], rk[0]); n1 = normed(qkv1, T1, rq[1], rk[1])
+    out0 = torch.zeros((B * max(T0, 1), C), device="cuda", dtype=torch.bfloat16)
+    out1 = torch.zeros((B * T1, C), device="cuda", dtype=torch.bfloat16)
+    if T0:
+        L.call("sd3_flash_attention_bf16", n0.data_ptr(), n1.data_ptr(), out0.data_ptr(), out1.data_ptr(), None, None, None, None, B, T0, T1, NH, HS, None)
+        parts = [n0.float().view(B, T0, 3, NH, HS), n1.float().view(B, T1, 3, NH, HS)]
+        got = torch.cat([out0.view(B, T0, C), out1.view(B, T1, C)], 1).float()
+    else:
+        L.call("sd3_flash_attention_bf16", n1.data_ptr(), None, out1.data_ptr(), None, None, None, None, None, B, T1, 0, NH, HS, None)
+        parts = [n1.float().view(B, T1, 3, NH, HS)]
+        got = out1.view(B, T1, C).float()
+    q, k, v = (torch.cat([p[:, :, i] for p in parts], 1).transpose(1, 2) for i in range(3))  # (B,NH,T,HS)
+    ref = (torch.softmax(q @ k.transpose(-1, -2) / 8.0, -1) @ v).transpose(1, 2).reshape(B, T0 + T1, C)
+    assert torch.isfinite(got).all()
+    assert rel_l2(host(got), host(ref)) <= 1e-2
+    assert float((got - ref).abs().max()) <= 0.05
+
+
 @pytest.mark.parametrize("case", ["overflow_mid", "overflow_to_inf", "first_tile_vanishes", "everything_vanishes", "harmless"])
 def test_flash_attention_bf16_fast_tiles_give_way_to_the_general_path(case):
     """Tiles in which no key is masked run with the softmax reference fixed at zero, as long as every lane's row sums stay between
