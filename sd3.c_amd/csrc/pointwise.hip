@@ -46,7 +46,9 @@ struct LnSegPair {
 template <typename OutT, int NV>
 __global__ void __launch_bounds__(256) ln_mod_vec_kernel(const LnSegPair<OutT> segs, float eps, int C) {
     const int lane = threadIdx.x & (WAVE - 1);
-    long long row = (long long)blockIdx.x * (blockDim.x / WAVE) + (threadIdx.x / WAVE);
+    // (the wavefront's index as a scalar: the row, the segment it belongs to and every pointer derived from them then live in scalar
+    // registers, which keeps the kernel within 64 vector registers, i.e. at 8 wavefronts per SIMD: all rows of the latent stream at once)
+    long long row = (long long)blockIdx.x * (blockDim.x / WAVE) + __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
     const int which = row >= segs.s[0].rows ? 1 : 0;
     if (which) row -= segs.s[0].rows;
     const LnSegDev<OutT>& g = segs.s[which];
