@@ -127,6 +127,36 @@ class PowerSampler:
                 "joules_per_step": round(avg * seconds / steps, 2)}
 
 
+def reference_api_rates(M, cfg, P, inputs, a, expect):
+    """The same forward through the entry points that keep the reference's argument list, i.e. receive the whole parameter map on
+    every call (DiT_forward, modules.cpp:1605-1613): `modules.DiT` of the Python mirror and, where it is built, `DiT_cuda` of the
+    compiled torch binding (tests/cpp). Both keep one context alive and re-use the bf16 weight copies while the map is unchanged."""
+    import torch
+    tail = (cfg.num_layers, set(cfg.dual_attention_layers), cfg.pooled_dim, cfg.captions_dim, cfg.in_channels, cfg.emb_dim, cfg.attn_heads,
+            cfg.mlp_expand, cfg.patch_size, cfg.pos_embed_max_size, cfg.base_height, cfg.use_qk_norm)
+    entries = [("modules.DiT", lambda: M.DiT(*inputs, P, *tail, precision=a.precision), M.release_shared_contexts)]
+    cpp = os.path.join(ROOT, "tests", "cpp")
+    if a.precision in ("bf16", "fp32") and os.path.exists(os.path.join(cpp, "sd3_ref_binding.so")):
+        sys.path.insert(0, cpp)
+        import sd3_ref_binding as F
+        F.set_precision(a.precision)
+        entries.append(("sd3_ref_binding.DiT_cuda", lambda: F.DiT_cuda(*inputs, P, *tail), F.release))
+    res = {}
+    for name, call, release in entries:
+        for _ in range(max(2, a.warmup)):
+            o = call()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(a.steps):
+            o = call()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        assert torch.equal(o, expect), name
+        release()
+        res[name] = {"value": round(a.steps / dt, 3), "unit": "steps/s", "ms_per_step": round(dt / a.steps * 1e3, 3)}
+    return res
+
+
 def mfma_probe():
     """What this device's matrix cores sustain on the instruction the GEMM and attention kernels use, issued back to back from
     registers by every wavefront (no memory traffic): with zero operands, and with random ones. The device holds its power
@@ -154,6 +184,7 @@ def main():
                     help="bf16 is the benchmark; the fp8 variants (MLP layers on the fp8 matrix instruction) do not meet its error criterion "
                          "and are for comparison only")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-reference-api", action="store_true", help="skip the timing through the reference-shaped entry points")
     ap.add_argument("--no-events", action="store_true", help="do not record per-kernel events during the timed steps")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one plain 1 GiB copy kernel (sd3::copy_rows_kernel), the known-size reference for scaling rocprofv3's "
@@ -218,6 +249,7 @@ def main():
         dt_prof = time.perf_counter() - t0
         prof = den.ctx.profile_end()
     assert torch.isfinite(out).all()
+    via_reference_api = None if a.no_reference_api else reference_api_rates(M, cfg, P, (pooled, captions, latent, timesteps), a, out)
 
     gemm_f, attn_f, embed_f = forward_flops(cfg, B, Tc, Tx)
     total_f = gemm_f + attn_f + embed_f
@@ -247,6 +279,10 @@ def main():
         "ms_per_step_profiled": round(dt_prof / a.steps * 1e3, 3) if dt_prof else None,
         "roofline": roofline, "kernels": kernels,
     }
+    if via_reference_api:
+        for v in via_reference_api.values():
+            v["ratio_to_value"] = round(v["value"] / res["value"], 4)
+        res["via_reference_api"] = via_reference_api
     res["power"] = power_stats
     if a.precision != "fp32":
         res["mfma_probe"] = mfma_probe()

@@ -37,7 +37,7 @@ typedef enum sd3_precision {
     SD3_PREC_BF16_FP8_TENSOR = 3
 } sd3_precision;
 
-typedef enum sd3_activation { SD3_ACT_SILU = 0, SD3_ACT_GELU_TANH = 1 } sd3_activation;
+typedef enum sd3_activation { SD3_ACT_SILU = 0, SD3_ACT_GELU_TANH = 1, SD3_ACT_GELU_ERF = 2 } sd3_activation;
 
 typedef struct sd3_ctx sd3_ctx; /* owns: bound weights table, bf16 weight copies, workspace, stream */
 
@@ -52,6 +52,9 @@ int sd3_layernorm(const float* x, float* y, float* mean, float* rstd, const floa
 int sd3_rmsnorm(const float* x, float* y, const float* w, float* rms, float eps, int B, int T, int C, void* stream);
 /* modules.cpp:192 rmsnorm_group: per-(token, group) RMSNorm over C/groups values with a shared weight of C/groups values. */
 int sd3_rmsnorm_group(const float* x, float* y, const float* w, float* rms, float eps, int groups, int B, int T, int C, void* stream);
+/* modules.cpp:280 gelu(x, y, n): the erf form 0.5 x (1 + erf(x / sqrt 2)), which the reference's extension exports as `gelu`
+ * (modules.cpp:1795). Not used by the forward path (the block MLPs use gelu_tanh). */
+int sd3_gelu(const float* in, float* out, long long n, void* stream);
 /* modules.cpp:293 gelu_tanh(input, output, n). */
 int sd3_gelu_tanh(const float* in, float* out, long long n, void* stream);
 /* modules.cpp:352 silu(x, y, n). */
@@ -111,13 +114,32 @@ int sd3_dit_block_w(sd3_ctx* ctx, const float* y, float* c, float* x, const sd3_
 
 int sd3_ctx_create(sd3_ctx** out, int device);
 int sd3_ctx_destroy(sd3_ctx* ctx);
+/* The stream that the context's calls enqueue on from now on (default: the null stream). The new stream is made to wait for
+ * the work of the context's earlier calls (they share the workspace and the derived weight copies) through an event the
+ * library records behind each call, so the previous stream may already have been destroyed by its owner. A stream must be
+ * alive while a call enqueues on it. Under stream capture no event is recorded or waited on: whoever replays a captured
+ * graph orders the replays against the context's other work. */
 int sd3_ctx_set_stream(sd3_ctx* ctx, void* stream);
 int sd3_ctx_synchronize(sd3_ctx* ctx);
 
 /* One entry of the reference's `name -> tensor` parameter map (modules.cpp:1512,1609). `ptr` is borrowed: it must stay
- * valid and unchanged while bound. Names are the reference's (modules.cpp:1558-1575, 1665-1728). */
+ * valid and unchanged while bound. Names are the reference's (modules.cpp:1558-1575, 1665-1728).
+ * The reference's entry points receive the whole map on every call (modules.cpp:1605-1613, 1783-1787); a caller shaped like
+ * them keeps one context and binds the map again each time: binding a name to the tensor it is already bound to (same
+ * address, same numel) is free and keeps the derived copies; a different address or size drops what was derived from the
+ * old tensor and from whatever lived at the new address before. What the library cannot see is a change of CONTENTS at an
+ * unchanged address (an in-place update, or memory that was freed and handed out again for another tensor of the same
+ * size): then call sd3_weights_forget(ptr) / sd3_weights_unbind(name) for that tensor, or sd3_weights_prepare for all. */
 int sd3_weights_bind(sd3_ctx* ctx, const char* name, const float* ptr, long long numel);
+/* Removes one name from the map (no error if it is not bound) and drops what was derived from its tensor. */
+int sd3_weights_unbind(sd3_ctx* ctx, const char* name);
+/* Drops the derived copies made from the tensor at `ptr` (its contents have changed); names stay bound, the copies are built
+ * again on next use. Also serves callers of sd3_dit_block_w, whose weights have no names. */
+int sd3_weights_forget(sd3_ctx* ctx, const float* ptr);
 int sd3_weights_clear(sd3_ctx* ctx);
+/* Number of derived weight copies the context has built since it was created (bf16 / fp8 / transposed copies, one per
+ * weight and kind): lets a caller or a test see whether a call re-used the existing copies or built new ones. */
+int sd3_weights_copies_built(sd3_ctx* ctx, long long* count);
 /* Rebuilds, from the current contents of the bound tensors, every derived copy a forward of `precision` uses (bf16: the
  * K-contiguous bf16 copies of the GEMM weights, the bf16 copies of the adaLN weights and of the patch-conv weight; fp32: the
  * transposed patch-conv weight). Optional before a first forward (copies are otherwise built on first use, inside that

@@ -21,6 +21,7 @@
 // ---- declarations of reference functions (external linkage in modules.cpp) ----
 void layernorm(float* x, float* y, float* mean, float* rstd, float* w, float* bias, float eps, int B, int T, int C);  // modules.cpp:10
 void rmsnorm_group(float* x, float* y, float* w, float* rms, float eps, int groups, int B, int T, int C);              // modules.cpp:192
+void gelu(float* x, float* y, long long n_elem);                                                                       // modules.cpp:280
 void gelu_tanh(float* input, float* output, long long n_elem);                                                         // modules.cpp:293
 void silu(float* x, float* y, long long n_elem);                                                                       // modules.cpp:352
 void linear(float* x, float* W, float* b, float* y, int B, int C_in, int C_out);                                       // modules.cpp:475
@@ -77,6 +78,7 @@ std::unordered_map<std::string, torch::Tensor> make_params(int n, const char** n
 REF_API void ref_layernorm(float* x, float* y, float eps, int B, int T, int C) { layernorm(x, y, nullptr, nullptr, nullptr, nullptr, eps, B, T, C); }
 REF_API void ref_rmsnorm_group(float* x, float* y, float* w, float eps, int groups, int B, int T, int C) { rmsnorm_group(x, y, w, nullptr, eps, groups, B, T, C); }
 REF_API void ref_gelu_tanh(float* in, float* out, long long n) { gelu_tanh(in, out, n); }
+REF_API void ref_gelu(float* in, float* out, long long n) { gelu(in, out, n); }
 REF_API void ref_silu(float* in, float* out, long long n) { silu(in, out, n); }
 REF_API void ref_linear(float* x, float* W, float* b, float* y, int B, int Cin, int Cout) { linear(x, W, b, y, B, Cin, Cout); }
 REF_API void ref_partial_linear(float* x, float* W, float* b, float* y, int M, int K, int N, int Nmax, int n0) { partial_linear(x, W, b, y, M, K, N, Nmax, n0); }

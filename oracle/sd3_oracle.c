@@ -56,6 +56,12 @@ void orc_gelu_tanh(const float* in, float* out, long n) {
     }
 }
 
+/* modules.cpp:280-285 (erf form, the extension's `gelu`): the division and erff are float, the outer product is double. */
+void orc_gelu(const float* in, float* out, long n) {
+    const float sqrt2 = sqrtf(2.0f);
+    for (long i = 0; i < n; i++) out[i] = (float)(0.5 * in[i] * (1.0 + erff(in[i] / sqrt2)));
+}
+
 /* modules.cpp:352-358 */
 void orc_silu(const float* in, float* out, long n) {
     for (long i = 0; i < n; i++) {

@@ -11,6 +11,7 @@
  *   orc_layernorm            torch.nn.functional.layer_norm; rows have mean 0 / variance 1
  *   orc_rmsnorm_heads        torch.nn.functional.rms_norm on the (rows, HS) view
  *   orc_gelu_tanh, orc_silu  torch gelu(approximate="tanh"), silu
+ *   orc_gelu                 torch gelu(approximate="none") (what module_tests/gelu.py:28 compares with); float64 closed form
  *   orc_linear, orc_partial_linear   x @ W + b in float64
  *   orc_attention            float64 softmax(QK^T/sqrt(HS))V; key-permutation invariance; ones-V
  *   orc_timestep_embedding   closed form cos/sin(t * 10000^(-i/128)) in float64
@@ -37,6 +38,8 @@ void orc_layernorm(const float* x, float* y, float eps, long rows, int C);
 void orc_rmsnorm_heads(float* x, const float* w, float eps, long rows, int HS);
 /* modules.cpp:293-300 */
 void orc_gelu_tanh(const float* in, float* out, long n);
+/* modules.cpp:280-285: 0.5 x (1 + erf(x / sqrt 2)), what the extension binds as `gelu` (modules.cpp:1795); not used by the forward path */
+void orc_gelu(const float* in, float* out, long n);
 /* modules.cpp:352-358 */
 void orc_silu(const float* in, float* out, long n);
 /* modules.cpp:475-490: y(M,N) = x(M,K) @ W(K,N) + b(N) */

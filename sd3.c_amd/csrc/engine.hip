@@ -73,13 +73,18 @@ static inline int fp8_kind(int prec) { return prec == SD3_PREC_BF16_FP8 ? 3 : pr
 struct sd3_ctx {
     int device = 0;
     hipStream_t stream = nullptr;
-    hipEvent_t order_event = nullptr;  // orders work across a change of stream (sd3_ctx_set_stream)
+    // Recorded behind the last kernel of every enqueueing call (outside stream capture). Everything that must wait for the
+    // context's earlier work between calls -- a change of stream, freeing derived copies, destroying the context -- waits on this
+    // event, which the library owns, and never touches the handle of a stream the caller may have destroyed since.
+    hipEvent_t order_event = nullptr;
+    bool order_pending = false;
     std::unordered_map<std::string, std::pair<const float*, long long>> params;
     std::map<std::pair<const float*, int>, PackedWeight> packed;
     std::map<std::tuple<int, int, int, int, int>, float*> pos_tables;  // (C, max, base, h, w) -> cropped table
     void* ws = nullptr;
     size_t ws_bytes = 0;
     void* static_scratch = nullptr;  // this device's address of the fixed scratch array (resolved when the context is created)
+    long long copies_built = 0;  // derived weight copies built so far (sd3_weights_copies_built)
     bool no_alloc = false;  // set for the duration of a call that must not allocate: a missing derived weight copy is then an error
     // optional per-kernel-class timing with HIP events on the context's stream
     bool prof_on = false;
@@ -119,6 +124,30 @@ struct Bump {
         off += bytes;
         return p;
     }
+};
+
+// Marks the end of an enqueueing call on the context's stream (see sd3_ctx::order_event). Nothing is recorded while the stream
+// is being captured into a graph: the event would become part of the capture, and replays are ordered by the caller.
+void record_order(sd3_ctx* ctx) {
+    if (!ctx->order_event) return;
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(ctx->stream, &cap) != hipSuccess) {
+        (void)hipGetLastError();
+        return;
+    }
+    if (cap != hipStreamCaptureStatusNone) return;
+    if (hipEventRecord(ctx->order_event, ctx->stream) == hipSuccess) ctx->order_pending = true;
+    else (void)hipGetLastError();
+}
+// Waits on the host until the work of every earlier call has finished (the device of the context must be current).
+int wait_idle(sd3_ctx* ctx) {
+    if (ctx->order_pending) SD3_HIP_TRY(hipEventSynchronize(ctx->order_event));
+    return SD3_OK;
+}
+struct OrderScope {  // records the order event when an enqueueing entry point returns, on every path
+    sd3_ctx* ctx;
+    explicit OrderScope(sd3_ctx* c) : ctx(c) {}
+    ~OrderScope() { record_order(ctx); }
 };
 
 int ensure_workspace(sd3_ctx* ctx, size_t bytes) {
@@ -172,6 +201,7 @@ int get_packed(sd3_ctx* ctx, const float* w, long long K, long long N, int kind,
         return rc;
     }
     ctx->packed[key] = p;
+    ctx->copies_built++;
     *out = p.ptr;
     return SD3_OK;
 }
@@ -184,7 +214,7 @@ int drop_packed_of(sd3_ctx* ctx, const float* w) {
         if (it == ctx->packed.end()) continue;
         if (!synced) {
             DeviceGuard g(ctx->device);
-            SD3_HIP_TRY(hipStreamSynchronize(ctx->stream));
+            SD3_TRY(wait_idle(ctx));
             synced = true;
         }
         DeviceGuard g(ctx->device);
@@ -473,7 +503,7 @@ int run_block(sd3_ctx* ctx, int prec, const float* y, float* c, float* x, const 
         } else {
             sets[n++] = joint;
         }
-        flop += 4.0 * B * d.NH * Tj * Tj * d.HS;
+        flop += 4.0 * B * d.NH * (d.discard ? (double)Tx : Tj) * Tj * d.HS;  // (a discard_context block computes no context queries)
         if (d.dual) {
             sets[n++] = dual_set;
             flop += 4.0 * B * d.NH * (double)Tx * Tx * d.HS;
@@ -485,7 +515,7 @@ int run_block(sd3_ctx* ctx, int prec, const float* y, float* c, float* x, const 
             wsp[n] = split_ws;
             n++;
         }
-        ProfScope ps(ctx, SD3_PROF_ATTENTION, flop, 1);
+        ProfScope ps(ctx, SD3_PROF_ATTENTION, flop, 1 + ((ctx_splits && !d.discard) ? 1 : 0));  // (+ the kernel that merges the key splits)
         SD3_TRY(attention_bf16_multi(sets, splits, wsp, n, B, d.NH, d.HS, st));  // q and k arrive normalised
     } else {
         SD3_TRY(attention(ctx, joint, B, d.NH, d.HS, bf));
@@ -650,6 +680,12 @@ int sd3_gelu_tanh(const float* in, float* out, long long n, void* stream) {
     NOTNULL(in); NOTNULL(out);
     return unary_op(in, out, n, SD3_ACT_GELU_TANH, ST(stream));
 }
+int sd3_gelu(const float* in, float* out, long long n, void* stream) {
+    SD3_REQUIRE(n >= 0, "gelu: negative size");
+    if (n == 0) return SD3_OK;
+    NOTNULL(in); NOTNULL(out);
+    return unary_op(in, out, n, SD3_ACT_GELU_ERF, ST(stream));
+}
 int sd3_silu(const float* in, float* out, long long n, void* stream) {
     SD3_REQUIRE(n >= 0, "silu: negative size");
     if (n == 0) return SD3_OK;
@@ -789,6 +825,10 @@ int sd3_ctx_create(sd3_ctx** out, int device) {
         // the address of the fixed scratch array on this device, asked for once per device with that device current
         DeviceGuard g(device);
         int rc = g.ok ? static_scratch_of(device, &c->static_scratch) : fail(SD3_ERR_HIP, "cannot select device %d", device);
+        if (rc == SD3_OK && hipEventCreateWithFlags(&c->order_event, hipEventDisableTiming) != hipSuccess) {
+            (void)hipGetLastError();
+            rc = fail(SD3_ERR_HIP, "ctx_create: cannot create the ordering event on device %d", device);
+        }
         if (rc != SD3_OK) {
             delete c;
             return rc;
@@ -800,7 +840,7 @@ int sd3_ctx_create(sd3_ctx** out, int device) {
 int sd3_weights_clear(sd3_ctx* ctx) {
     NOTNULL(ctx);
     DeviceGuard g(ctx->device);
-    SD3_HIP_TRY(hipStreamSynchronize(ctx->stream));
+    SD3_TRY(wait_idle(ctx));
     for (auto& kv : ctx->packed) (void)hipFree(kv.second.ptr);
     ctx->packed.clear();
     ctx->params.clear();
@@ -810,7 +850,7 @@ int sd3_ctx_destroy(sd3_ctx* ctx) {
     if (!ctx) return SD3_OK;
     {
         DeviceGuard g(ctx->device);
-        (void)hipStreamSynchronize(ctx->stream);
+        (void)wait_idle(ctx);
         for (auto& kv : ctx->packed) (void)hipFree(kv.second.ptr);
         for (auto& kv : ctx->pos_tables) (void)hipFree(kv.second);
         if (ctx->ws) (void)hipFree(ctx->ws);
@@ -830,15 +870,15 @@ int sd3_ctx_set_stream(sd3_ctx* ctx, void* stream) {
     if (ST(stream) == ctx->stream) return SD3_OK;
     // The workspace, the derived weight copies and the position tables are shared by everything the context enqueues: work
     // already queued on the old stream must finish before work on the new stream touches them.
+    // The old stream's handle is not used here (its owner may have destroyed it since the last call): the new stream waits on the
+    // event recorded behind that call's last kernel. A stream that is being captured into a graph cannot wait on work outside the
+    // capture; its owner has ordered the capture behind earlier work, and orders the graph's replays.
     DeviceGuard g(ctx->device);
     if (!g.ok) return fail(SD3_ERR_HIP, "cannot select device %d", ctx->device);
-    if (!ctx->order_event) SD3_HIP_TRY(hipEventCreateWithFlags(&ctx->order_event, hipEventDisableTiming));
-    if (hipEventRecord(ctx->order_event, ctx->stream) == hipSuccess) {
-        SD3_HIP_TRY(hipStreamWaitEvent(ST(stream), ctx->order_event, 0));
-    } else {
-        // the old stream no longer exists (its owner destroyed it): whatever ran on it is ordered by a device-wide wait instead
-        (void)hipGetLastError();
-        SD3_HIP_TRY(hipDeviceSynchronize());
+    if (ctx->order_pending) {
+        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+        SD3_HIP_TRY(hipStreamIsCapturing(ST(stream), &cap));
+        if (cap == hipStreamCaptureStatusNone) SD3_HIP_TRY(hipStreamWaitEvent(ST(stream), ctx->order_event, 0));
     }
     ctx->stream = ST(stream);
     return SD3_OK;
@@ -853,12 +893,32 @@ int sd3_weights_bind(sd3_ctx* ctx, const char* name, const float* ptr, long long
     NOTNULL(ctx); NOTNULL(name); NOTNULL(ptr);
     SD3_REQUIRE(numel > 0, "weights_bind(%s): numel must be positive", name);
     SD3_REQUIRE((reinterpret_cast<uintptr_t>(ptr) & 3) == 0, "weights_bind(%s): pointer is not 4-byte aligned", name);
-    // derived copies are keyed by the tensor's address: what was made from the tensor this name was bound to before, or from
-    // an earlier tensor that lived at the new address, must not survive the re-binding
+    // Binding a name again to the tensor it is already bound to (same address, same size) changes nothing and keeps the derived
+    // copies: callers shaped like the reference's entry points hand over the whole parameter map on every call.
     auto old = ctx->params.find(name);
+    if (old != ctx->params.end() && old->second.first == ptr && old->second.second == numel) return SD3_OK;
+    // Otherwise: derived copies are keyed by the tensor's address, so what was made from the tensor this name was bound to before,
+    // or from an earlier tensor that lived at the new address, must not survive the re-binding.
     if (old != ctx->params.end() && old->second.first != ptr) SD3_TRY(drop_packed_of(ctx, old->second.first));
     SD3_TRY(drop_packed_of(ctx, ptr));
     ctx->params[name] = std::make_pair(ptr, numel);
+    return SD3_OK;
+}
+int sd3_weights_unbind(sd3_ctx* ctx, const char* name) {
+    NOTNULL(ctx); NOTNULL(name);
+    auto it = ctx->params.find(name);
+    if (it == ctx->params.end()) return SD3_OK;
+    SD3_TRY(drop_packed_of(ctx, it->second.first));
+    ctx->params.erase(it);
+    return SD3_OK;
+}
+int sd3_weights_forget(sd3_ctx* ctx, const float* ptr) {
+    NOTNULL(ctx); NOTNULL(ptr);
+    return drop_packed_of(ctx, ptr);
+}
+int sd3_weights_copies_built(sd3_ctx* ctx, long long* count) {
+    NOTNULL(ctx); NOTNULL(count);
+    *count = ctx->copies_built;
     return SD3_OK;
 }
 int sd3_weights_prepare(sd3_ctx* ctx, int precision) {
@@ -867,7 +927,8 @@ int sd3_weights_prepare(sd3_ctx* ctx, int precision) {
     DeviceGuard g(ctx->device);
     if (!g.ok) return fail(SD3_ERR_HIP, "cannot select device %d", ctx->device);
     // drop what exists (the bound tensors may have been changed in place) ...
-    SD3_HIP_TRY(hipStreamSynchronize(ctx->stream));
+    OrderScope order(ctx);
+    SD3_TRY(wait_idle(ctx));
     for (auto& kv : ctx->packed) (void)hipFree(kv.second.ptr);
     ctx->packed.clear();
     // ... and rebuild every copy the forward of this precision would otherwise build on first use. A linear layer's shape follows
@@ -945,6 +1006,7 @@ int sd3_dit_block_w(sd3_ctx* ctx, const float* y, float* c, float* x, const sd3_
     if (Tc > 0) NOTNULL(c);
     DeviceGuard g(ctx->device);
     if (!g.ok) return fail(SD3_ERR_HIP, "cannot select device %d", ctx->device);
+    OrderScope order(ctx);
     SD3_TRY(ensure_workspace(ctx, block_workspace_bytes(d, precision)));
     Bump ws(ctx->ws, ctx->ws_bytes);
     return run_block(ctx, precision, y, c, x, *w, d, nullptr, nullptr, ws);
@@ -980,6 +1042,7 @@ int sd3_dit_block_static(sd3_ctx* ctx, const float* y, float* c, float* x, const
     DeviceGuard g(ctx->device);
     if (!g.ok) return fail(SD3_ERR_HIP, "cannot select device %d", ctx->device);
     if (!ctx->static_scratch) return fail(SD3_ERR_HIP, "dit_block_static: the fixed scratch array has no address on device %d", ctx->device);
+    OrderScope order(ctx);  // (records an event that exists since the context was created: no allocation)
     Bump ws(ctx->static_scratch, SD3_STATIC_SCRATCH_BYTES);
     ctx->no_alloc = true;
     const int rc = run_block(ctx, precision, y, c, x, w, d, nullptr, nullptr, ws);
@@ -1011,6 +1074,7 @@ static int dit_forward_impl(sd3_ctx* ctx, const float* pooled, const float* capt
     if (bf && ((captions_dim % 64) || (Kp % 64))) return fail(SD3_ERR_UNSUPPORTED, "bf16 path needs captions_dim and C_in*patch^2 to be multiples of 64");
     DeviceGuard g(ctx->device);
     if (!g.ok) return fail(SD3_ERR_HIP, "cannot select device %d", ctx->device);
+    OrderScope order(ctx);
     hipStream_t st = ctx->stream;
 
     std::vector<char> is_dual(num_layers, 0);

@@ -42,6 +42,8 @@ inline void rmsnorm(float* x, float* y, float* w, float* rms, float eps, int B, 
 inline void rmsnorm_group(float* x, float* y, float* w, float* rms, float eps, int groups, int B, int T, int C) {
     sd3::check(sd3_rmsnorm_group(x, y, w, rms, eps, groups, B, T, C, sd3::modules_stream()));
 }
+// modules.cpp:280 (erf form)
+inline void gelu(float* x, float* y, long long n_elem) { sd3::check(sd3_gelu(x, y, n_elem, sd3::modules_stream())); }
 // modules.cpp:293
 inline void gelu_tanh(float* input, float* output, long long n_elem) { sd3::check(sd3_gelu_tanh(input, output, n_elem, sd3::modules_stream())); }
 // modules.cpp:352
@@ -113,6 +115,12 @@ inline void split_along_tokens(float* input, float* split1, float* split2, int B
 
 // modules.cpp:1340-1365, same 49 pointers and 9 scalars in the same order. The 16 scratch pointers are accepted for
 // source compatibility and not used: the library keeps its own (differently shaped) workspace in the context.
+//
+// WARNING for SD3_PREC_BF16: the bf16 copies of the weight matrices are made on first use and kept in the context, KEYED BY THE
+// WEIGHT'S DEVICE ADDRESS. Raw pointers carry no notion of "changed": a caller that overwrites a weight buffer in place, or frees
+// it and gets the same address back for other weights, must call sd3_weights_prepare(sd3::modules_ctx(), SD3_PREC_BF16) (drops
+// and rebuilds every copy of the bound names) or sd3_weights_forget(sd3::modules_ctx(), ptr) for that buffer before the next
+// dit_block, or the block runs on the old copies. SD3_PREC_F32 reads the weights in place and has no such state.
 inline void dit_block(float* y, float* c, float* x,
                       float* c_ada_lnorm_weights, float* c_ada_lnorm_biases, float* c_Wqkv, float* c_bias_qkv, float* c_rms_Wq, float* c_rms_Wk,
                       float* c_Wout, float* c_bias_out, float* c_mlp_W1, float* c_mlp_b1, float* c_mlp_W2, float* c_mlp_b2,

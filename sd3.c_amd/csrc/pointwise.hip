@@ -255,11 +255,14 @@ int rmsnorm_rows(const float* x, float* y, const float* w, float* rms, float eps
 }
 
 // ---- elementwise ----
-template <int OP>  // 0 silu, 1 gelu_tanh
+template <int OP>  // 0 silu, 1 gelu_tanh, 2 gelu (erf form, modules.cpp:280-285)
 __global__ void __launch_bounds__(256) unary_kernel(const float* __restrict__ in, float* __restrict__ out, long long n) {
     long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     const long long stride = (long long)gridDim.x * blockDim.x;
-    for (; i < n; i += stride) out[i] = (OP == 0) ? silu_precise(in[i]) : gelu_tanh_precise(in[i]);
+    for (; i < n; i += stride) {
+        const float v = in[i];
+        out[i] = (OP == 0) ? silu_precise(v) : (OP == 1) ? gelu_tanh_precise(v) : 0.5f * v * (1.0f + erff(v * 0.70710678118654752f));
+    }
 }
 static unsigned grid_for(long long n, int per_block = 256, unsigned cap = 256 * 64) {
     long long g = (n + per_block - 1) / per_block;
@@ -268,6 +271,7 @@ static unsigned grid_for(long long n, int per_block = 256, unsigned cap = 256 * 
 int unary_op(const float* in, float* out, long long n, int act, hipStream_t st) {
     if (n == 0) return SD3_OK;
     if (act == SD3_ACT_SILU) hipLaunchKernelGGL((unary_kernel<0>), dim3(grid_for(n)), dim3(256), 0, st, in, out, n);
+    else if (act == SD3_ACT_GELU_ERF) hipLaunchKernelGGL((unary_kernel<2>), dim3(grid_for(n)), dim3(256), 0, st, in, out, n);
     else hipLaunchKernelGGL((unary_kernel<1>), dim3(grid_for(n)), dim3(256), 0, st, in, out, n);
     return launch_status("activation");
 }

@@ -57,7 +57,8 @@ def _host_op(fn):
 
 layer_norm = _host_op(lambda input, weight=None, bias=None, eps=1e-5, save_for_backward=False: _M.layer_norm(input, weight, bias, eps, save_for_backward))
 rms_norm = _host_op(lambda input, weight, eps, save_for_backward=False: _M.rms_norm(input, weight, eps, save_for_backward))
-gelu = _host_op(_M.gelu_tanh)
+gelu = _host_op(_M.gelu)            # modules.cpp:1795 binds `gelu` to the erf form (modules.cpp:280-285)
+gelu_tanh = _host_op(_M.gelu_tanh)  # the block MLPs' activation (modules.cpp:293); not exported by the reference's extension, kept under its own name
 silu = _host_op(_M.silu)
 linear = _host_op(_M.linear)
 conv2d = _host_op(_M.conv2d)

@@ -18,6 +18,7 @@ SIGNATURES = {
     "sd3_layernorm": [vp, vp, vp, vp, vp, vp, cf, ci, ci, ci, vp],
     "sd3_rmsnorm": [vp, vp, vp, vp, cf, ci, ci, ci, vp],
     "sd3_rmsnorm_group": [vp, vp, vp, vp, cf, ci, ci, ci, ci, vp],
+    "sd3_gelu": [vp, vp, cll, vp],
     "sd3_gelu_tanh": [vp, vp, cll, vp],
     "sd3_silu": [vp, vp, cll, vp],
     "sd3_linear": [vp, vp, vp, vp, ci, ci, ci, vp],
@@ -40,7 +41,10 @@ SIGNATURES = {
     "sd3_ctx_set_stream": [vp, vp],
     "sd3_ctx_synchronize": [vp],
     "sd3_weights_bind": [vp, cs, vp, cll],
+    "sd3_weights_unbind": [vp, cs],
+    "sd3_weights_forget": [vp, vp],
     "sd3_weights_clear": [vp],
+    "sd3_weights_copies_built": [vp, C.POINTER(cll)],
     "sd3_weights_prepare": [vp, ci],
     "sd3_dit_block": [vp, vp, vp, vp, cs] + [ci] * 10,
     "sd3_dit_block_static": [vp, vp, vp, vp, cs] + [ci] * 10,

@@ -62,6 +62,14 @@ def rms_norm_group(input, weight, eps, groups):
     return y
 
 
+def gelu(input):
+    """modules.cpp:302 GELU_forward: the erf form (modules.cpp:280-285), what the extension exports as `gelu`."""
+    x = _dev(input, "input")
+    y = torch.empty_like(x)
+    L.call("sd3_gelu", _p(x), _p(y), x.numel(), _stream())
+    return y
+
+
 def gelu_tanh(input):
     """modules.cpp:293 gelu_tanh (the activation of the block MLPs)."""
     x = _dev(input, "input")
@@ -223,10 +231,38 @@ class Context:
         self._keep = {}
 
     def bind(self, params):
+        """Adds `params` to the bound map. A name that is already bound to the same tensor (same storage address and size, unchanged
+        torch version counter) costs nothing and keeps the library's derived copies; a tensor that torch has modified in place
+        since it was bound has its copies dropped; anything else is bound anew."""
+        keep = self._keep
         for name, t in params.items():
+            old = keep.get(name)
+            if old is not None:
+                ot, over = old
+                if ot is t or (ot.data_ptr() == t.data_ptr() and ot.numel() == t.numel()):
+                    if t._version != over:  # same memory, new contents
+                        L.call("sd3_weights_forget", self._h, _p(t))
+                        keep[name] = (t, t._version)
+                    elif ot is not t:
+                        keep[name] = (t, over)
+                    continue
             _dev(t, name)
             L.call("sd3_weights_bind", self._h, name.encode(), _p(t), t.numel())
-            self._keep[name] = t
+            keep[name] = (t, t._version)  # the reference keeps the address alive (and out of the allocator's hands) while bound
+
+    def set_params(self, params):
+        """Makes the bound map equal to `params` (the reference's entry points receive the whole map on every call, modules.cpp:1512,
+        1609): names that are not in it are unbound, the rest goes through `bind`, so an unchanged map keeps every derived copy."""
+        for name in [n for n in self._keep if n not in params]:
+            L.call("sd3_weights_unbind", self._h, name.encode())
+            del self._keep[name]
+        self.bind(params)
+
+    def copies_built(self):
+        """Derived weight copies (bf16 / fp8 / transposed) built by this context so far."""
+        n = C.c_longlong(0)
+        L.call("sd3_weights_copies_built", self._h, C.byref(n))
+        return n.value
 
     def clear(self):
         L.call("sd3_weights_clear", self._h)
@@ -313,18 +349,37 @@ class Context:
             pass
 
 
+_shared = {}  # device index -> the Context behind the reference-shaped entry points below
+
+
+def shared_context(device):
+    """The one context per device that `Dit_block`, `DiT_block_cuda` and `DiT` run in. The reference's entry points take the parameter
+    map on every call and keep nothing between calls; here the context stays alive, each call hands its map to `set_params`, and a
+    map that has not changed re-uses the bf16 weight copies and the workspace of the previous call. The context keeps the last
+    map's tensors alive until the next call replaces them or `release_shared_contexts()` is called."""
+    idx = torch.device(device).index
+    idx = torch.cuda.current_device() if idx is None else idx
+    ctx = _shared.get(idx)
+    if ctx is None:
+        ctx = _shared[idx] = Context(idx)
+    return ctx
+
+
+def release_shared_contexts():
+    """Destroys the contexts behind `Dit_block` / `DiT` (bf16 copies, workspaces, references to the last parameter maps)."""
+    for ctx in _shared.values():
+        ctx.close()
+    _shared.clear()
+
+
 def Dit_block(temp_embeddings, context_embeddings, latent_vector, params, B, Tc, Tx, emb_dim, attn_heads, mlp_expand, use_dual_attention, use_qk_norm,
               discard_context, precision="fp32"):
-    """modules.cpp:1508 DiT_block_forward: mutates and returns [context_embeddings, latent_vector]."""
-    ctx = Context(latent_vector.device)
-    try:
-        ctx.bind(params)
-        out = ctx.block(temp_embeddings, context_embeddings, latent_vector, B, Tc, Tx, emb_dim, attn_heads, mlp_expand, use_dual_attention, use_qk_norm,
-                        discard_context, precision)
-        ctx.synchronize()
-        return out
-    finally:
-        ctx.close()
+    """modules.cpp:1508 DiT_block_forward: mutates and returns [context_embeddings, latent_vector]. Enqueued on torch's current
+    stream; like the reference's GPU entry it does not wait for the result (cuda/dit.cu:1060)."""
+    ctx = shared_context(latent_vector.device)
+    ctx.set_params(params)
+    return ctx.block(temp_embeddings, context_embeddings, latent_vector, B, Tc, Tx, emb_dim, attn_heads, mlp_expand, use_dual_attention, use_qk_norm,
+                     discard_context, precision)
 
 
 def DiT_block_cuda(*args, **kwargs):
@@ -334,16 +389,12 @@ def DiT_block_cuda(*args, **kwargs):
 
 def DiT(pooled_captions, captions, latent_vector, timesteps, params, num_layers, dual_attention_layers, pooled_dim, captions_dim, C_in, emb_dim,
         attn_heads, mlp_expand, patch_size, pos_embed_max_size, base_height, use_qk_norm, precision="fp32"):
-    """modules.cpp:1605 DiT_forward: returns a new (B, C_in, H, W) tensor; inputs are left untouched."""
-    ctx = Context(latent_vector.device)
-    try:
-        ctx.bind(params)
-        out = ctx.forward(pooled_captions, captions, latent_vector, timesteps, num_layers, dual_attention_layers, pooled_dim, captions_dim, C_in, emb_dim,
-                          attn_heads, mlp_expand, patch_size, pos_embed_max_size, base_height, use_qk_norm, precision)
-        ctx.synchronize()
-        return out
-    finally:
-        ctx.close()
+    """modules.cpp:1605 DiT_forward: returns a new (B, C_in, H, W) tensor; inputs are left untouched. Enqueued on torch's current
+    stream, in the shared per-device context (see `shared_context`)."""
+    ctx = shared_context(latent_vector.device)
+    ctx.set_params(params)
+    return ctx.forward(pooled_captions, captions, latent_vector, timesteps, num_layers, dual_attention_layers, pooled_dim, captions_dim, C_in, emb_dim,
+                       attn_heads, mlp_expand, patch_size, pos_embed_max_size, base_height, use_qk_norm, precision)
 
 
 class Denoiser:

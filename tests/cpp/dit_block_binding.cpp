@@ -17,13 +17,43 @@
 static sd3_ctx* g_ctx = nullptr;
 static int g_precision = SD3_PREC_F32;
 
+// The reference's entry points receive the parameter map on every call. The context lives across calls and the incoming map is
+// compared with the one bound by the previous call: an unchanged entry costs a hash lookup and keeps the library's bf16 copy of
+// that weight; an entry whose tensor torch has modified in place (version counter) has its copies dropped; a new or moved
+// tensor is bound; a name that is gone is unbound. The previous map's tensors are held until then, so that their addresses
+// cannot be handed out again for other data in the meantime.
+struct Bound {
+    torch::Tensor t;
+    uint32_t version;
+};
+static std::unordered_map<std::string, Bound> g_bound;
+
+static void ok(int rc) {
+    if (rc != SD3_OK) throw std::runtime_error(sd3_last_error());
+}
 static void bind_all(std::unordered_map<std::string, torch::Tensor>& params, const torch::Tensor& like) {
-    if (!g_ctx && sd3_ctx_create(&g_ctx, like.get_device()) != SD3_OK) throw std::runtime_error(sd3_last_error());
-    sd3_ctx_set_stream(g_ctx, c10::hip::getCurrentHIPStream().stream());
-    sd3_weights_clear(g_ctx);  // the map may differ from the previous call's
-    for (auto& kv : params)    // same names as get_ptr() looks up, modules.cpp:1558-1575
-        if (sd3_weights_bind(g_ctx, kv.first.c_str(), kv.second.data_ptr<float>(), kv.second.numel()) != SD3_OK)
-            throw std::runtime_error(sd3_last_error());
+    if (!g_ctx) ok(sd3_ctx_create(&g_ctx, like.get_device()));
+    ok(sd3_ctx_set_stream(g_ctx, c10::hip::getCurrentHIPStream().stream()));
+    for (auto it = g_bound.begin(); it != g_bound.end();) {
+        if (params.find(it->first) == params.end()) {
+            ok(sd3_weights_unbind(g_ctx, it->first.c_str()));
+            it = g_bound.erase(it);
+        } else {
+            ++it;
+        }
+    }
+    for (auto& kv : params) {  // same names as get_ptr() looks up, modules.cpp:1558-1575
+        const torch::Tensor& t = kv.second;
+        const float* p = t.data_ptr<float>();
+        const uint32_t version = t._version();
+        auto old = g_bound.find(kv.first);
+        if (old != g_bound.end() && old->second.t.data_ptr<float>() == p && old->second.t.numel() == t.numel()) {
+            if (old->second.version != version) ok(sd3_weights_forget(g_ctx, p));  // same memory, new contents
+        } else {
+            ok(sd3_weights_bind(g_ctx, kv.first.c_str(), p, t.numel()));
+        }
+        g_bound[kv.first] = Bound{t, version};
+    }
 }
 
 std::vector<torch::Tensor> DiT_block_forward_cuda(torch::Tensor& temp_embeddings, torch::Tensor& context_embeddings, torch::Tensor& latent_vector,
@@ -56,8 +86,14 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("DiT_block_cuda", &DiT_block_forward_cuda, "DiT block forward on the GPU (modules.cpp:1814)");
     m.def("DiT_cuda", &DiT_forward_cuda, "DiT forward on the GPU (argument list of modules.cpp:1811)");
     m.def("set_precision", [](const std::string& p) { g_precision = p == "bf16" ? SD3_PREC_BF16 : SD3_PREC_F32; });
+    m.def("copies_built", []() {
+        long long n = 0;
+        if (g_ctx) ok(sd3_weights_copies_built(g_ctx, &n));
+        return n;
+    }, "derived weight copies the binding's context has built so far");
     m.def("release", []() {
         if (g_ctx) sd3_ctx_destroy(g_ctx);
         g_ctx = nullptr;
+        g_bound.clear();
     });
 }

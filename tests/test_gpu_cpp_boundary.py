@@ -102,3 +102,72 @@ def test_reference_side_torch_binding_block_and_forward():
     finally:
         F.set_precision("fp32")
         F.release()
+
+
+def _dit_args(k):
+    cfg = k["cfg"]
+    tail = (cfg.num_layers, set(cfg.dual_attention_layers), cfg.pooled_dim, cfg.captions_dim, cfg.in_channels, cfg.emb_dim, cfg.attn_heads, cfg.mlp_expand,
+            cfg.patch_size, cfg.pos_embed_max_size, cfg.base_height, cfg.use_qk_norm)
+    return [torch.from_numpy(k[n]).cuda() for n in ("pooled", "captions", "latent", "timesteps")], tail
+
+
+def _reference_shaped_calls_keep_copies(call, copies_built, release):
+    """`call(params)` is an entry point with the reference's argument list (the whole parameter map on every call, modules.cpp:1605-1613,
+    1783-1787). With an unchanged map the second call must build no weight copy; a tensor changed in place through torch, a tensor
+    replaced by another one, and a name that disappears must all be seen. Expected outputs come from a released (empty) context."""
+    k = cases.dit_case("dit_hs64")
+    params = {n: torch.from_numpy(v).cuda() for n, v in k["params"].items()}
+
+    def fresh(p):
+        release()
+        out = call(p).clone()
+        release()
+        return out
+
+    out1 = call(params)
+    n1 = copies_built()
+    assert n1 > 0                                       # the bf16 path works on derived copies
+    out2 = call(params)
+    assert copies_built() == n1 and torch.equal(out1, out2)   # same map: nothing rebuilt, same result
+    assert rel_l2(out1.cpu().numpy(), GOLDEN["dit_hs64.out"]) <= BF16_REL_L2
+    name = "transformer.0.latent_mlp.lin2.weight"
+    params[name].mul_(1.5)                              # in place, through torch: the version counter moves
+    out3 = call(params)
+    assert copies_built() == n1 + 1 and not torch.equal(out3, out1)
+    name2 = "transformer.1.latent_to_qkv.weight"
+    params[name2] = (params[name2] * 0.5).contiguous()  # another tensor under the same name
+    out4 = call(params)
+    assert copies_built() == n1 + 2 and not torch.equal(out4, out3)
+    want = fresh(params)
+    assert torch.equal(out4, want)                      # exactly what a context that has never seen the old tensors computes
+    call(params)
+    n5 = copies_built()
+    missing = {n: t for n, t in params.items() if n != "transformer.0.latent_dual_to_qkv.weight"}
+    with pytest.raises(Exception):
+        call(missing)                                   # a name that is gone from the map is gone from the context
+        torch.cuda.synchronize()
+    assert torch.equal(call(params), want) and copies_built() == n5 + 1   # (only that weight's copy is built again)
+    release()
+
+
+def test_binding_keeps_weight_copies_across_reference_shaped_calls():
+    F = _binding()
+    k = cases.dit_case("dit_hs64")
+    args, tail = _dit_args(k)
+    try:
+        F.set_precision("bf16")
+        _reference_shaped_calls_keep_copies(lambda p: F.DiT_cuda(*args, p, *tail), F.copies_built, F.release)
+    finally:
+        F.set_precision("fp32")
+        F.release()
+
+
+def test_python_mirror_keeps_weight_copies_across_reference_shaped_calls():
+    from gpu_util import M
+    k = cases.dit_case("dit_hs64")
+    args, tail = _dit_args(k)
+    try:
+        _reference_shaped_calls_keep_copies(lambda p: M.DiT(*args, p, *tail, precision="bf16"),
+                                            lambda: M.shared_context(args[2].device).copies_built(), M.release_shared_contexts)
+    finally:
+        M.release_shared_contexts()

@@ -52,6 +52,12 @@ def test_activations():
     ol.oracle().orc_silu(fp(x), fp(s), x.size)
     assert max_abs(host(M.gelu_tanh(dev(x))), g) <= 1e-5
     assert max_abs(host(M.silu(dev(x))), s) <= 1e-5
+    # the erf form, which the reference's extension calls `gelu` (modules.cpp:1795; module_tests/gelu.py:28 holds it to torch's
+    # gelu(approximate="none")); 1e-5 separates it from the tanh form (up to ~5e-4 apart)
+    e = np.empty_like(x)
+    ol.oracle().orc_gelu(fp(x), fp(e), x.size)
+    assert max_abs(host(M.gelu(dev(x))), e) <= 1e-5
+    assert max_abs(e, torch.nn.functional.gelu(torch.from_numpy(x).double(), approximate="none").numpy()) <= 1e-6
 
 
 @pytest.mark.parametrize("Mr,K,N", [(7, 40, 33), (1, 5, 3), (130, 320, 260), (64, 256, 128), (2, 1536, 64), (300, 64, 1536), (129, 17, 131)])

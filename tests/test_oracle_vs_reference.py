@@ -33,7 +33,7 @@ def test_primitives_bit_exact():
     r.ref_rmsnorm_group(fp(b), fp(b), fp(w), C.c_float(1e-6), 3, 1, 6, 96)
     assert np.array_equal(a, b)
     v = randn(4096) * 4
-    for of, rf in ((o.orc_gelu_tanh, r.ref_gelu_tanh), (o.orc_silu, r.ref_silu)):
+    for of, rf in ((o.orc_gelu_tanh, r.ref_gelu_tanh), (o.orc_silu, r.ref_silu), (o.orc_gelu, r.ref_gelu)):
         a, b = np.empty_like(v), np.empty_like(v)
         of(fp(v), fp(a), 4096)
         rf(fp(v), fp(b), C.c_longlong(4096))

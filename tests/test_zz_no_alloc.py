@@ -56,3 +56,41 @@ def test_static_block_refuses_what_does_not_fit_and_unprepared_bf16_weights():
         assert e.value.status == 3 and "fixed scratch" in str(e.value)
     finally:
         ctx.close()
+
+
+@pytest.mark.parametrize("precision", ["fp32", "bf16"])
+def test_static_block_leaves_device_memory_alone_with_profiling_on_and_under_graph_capture(precision):
+    """What "allocates nothing" means, observed: the device's free memory (hipMemGetInfo) is the same before and after a call, also
+    while the library's per-kernel profiling is switched on (which otherwise creates events), and the call can be captured into a HIP
+    graph -- where an allocation would fail -- whose replays give the bits of sd3_dit_block."""
+    import torch
+    C, NH = 128, 2
+    params = dev_params(synthetic_params_numpy(block_param_shapes(C, 4, True, True, False, C // NH), 79, 0.1, 0.1))
+    ctx = M.Context()
+    try:
+        ctx.bind(params)
+        k = _case(2, 9, 300, C, NH, 9)
+        args = (k["B"], k["Tc"], k["Tx"], k["C"], k["NH"], 4, k["dual"], True, k["discard"])
+        cw, xw = _run(ctx, k, precision, static=False)   # (also builds the bf16 weight copies)
+        y, c, x = dev(k["y"]), dev(k["c"]), dev(k["x"])
+        c0, x0 = c.clone(), x.clone()
+        torch.cuda.synchronize()
+        free_before = torch.cuda.mem_get_info()[0]
+        ctx.profile_begin()
+        ctx.block_static(y, c, x, *args, precision=precision)
+        prof = ctx.profile_end()                          # (waits for the stream)
+        assert torch.cuda.mem_get_info()[0] == free_before
+        assert all(n == 0 for _, _, n in prof.values())   # no event was created or recorded for this call
+        assert np.array_equal(host(c), cw) and np.array_equal(host(x), xw)
+        graph, side = torch.cuda.CUDAGraph(), torch.cuda.Stream()
+        c.copy_(c0); x.copy_(x0)
+        torch.cuda.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            ctx.block_static(y, c, x, *args, precision=precision)
+        for _ in range(3):                                # every replay, with eager work and synchronisations in between
+            c.copy_(c0); x.copy_(x0)
+            torch.cuda.synchronize()
+            graph.replay()
+            assert np.array_equal(host(c), cw) and np.array_equal(host(x), xw)
+    finally:
+        ctx.close()
