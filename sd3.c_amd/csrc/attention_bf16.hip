@@ -29,8 +29,20 @@ constexpr int BQ = NW * QW;      // queries per workgroup
 constexpr int BKV = 64;          // keys per tile
 constexpr int K_BYTES = BKV * 128, V_BYTES = BKV * 128, STAGE_BYTES = K_BYTES + V_BYTES;
 constexpr int O_PITCH = 72;      // bf16 per staged output row
-constexpr int NSTAGE = 3;
-constexpr int SMEM_BYTES = (NSTAGE * STAGE_BYTES > NW * QW * O_PITCH * 2) ? NSTAGE * STAGE_BYTES : NW * QW * O_PITCH * 2;
+// Tiles are requested PF tiles ahead of the one being worked on, into a ring of PF + 2 LDS stages (the tile in use, PF on their
+// way or landed, and the stage of the tile before, which the newest request overwrites). One tile ahead is enough: with two
+// (SD3_ATTN_PREFETCH_2; not with the K rows passing through registers, NORM) and the barrier waiting only for the tile it
+// publishes, nothing was gained at any occupancy (measured), so the wait in the middle of a tile is not where time goes.
+constexpr int prefetch_tiles(bool norm) {
+#ifdef SD3_ATTN_PREFETCH_2
+    return norm ? 1 : 2;
+#else
+    return 1;
+#endif
+}
+constexpr int smem_bytes(bool norm) {
+    return ((prefetch_tiles(norm) + 2) * STAGE_BYTES > NW * QW * O_PITCH * 2) ? (prefetch_tiles(norm) + 2) * STAGE_BYTES : NW * QW * O_PITCH * 2;
+}
 
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 typedef const __attribute__((address_space(1))) void* glb_ptr_t;
@@ -86,6 +98,20 @@ __device__ __forceinline__ uint2 lds_read_tr16_b64(uint32_t lds_byte_addr, int i
     asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(r) : "v"(lds_byte_addr), "i"(imm_offset));
     return r;
 }
+// A plain 16-byte LDS read issued the same way (K fragments in the hand-ordered steps of the fast tiles), and the waits that name
+// what has landed: LDS operations return in order, so "at most N outstanding" means all but the newest N have arrived.
+__device__ __forceinline__ bf16x8_t lds_read_b128(uint32_t lds_byte_addr, int imm_offset) {
+    bf16x8_t r;
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r) : "v"(lds_byte_addr), "i"(imm_offset));
+    return r;
+}
+template <int N>
+__device__ __forceinline__ void lds_wait_k(bf16x8_t (&k)[4]) {
+    static_assert(N == 0 || N == 4 || N == 8, "outstanding LDS reads behind the four K fragments");
+    if (N == 8) asm volatile("s_waitcnt lgkmcnt(8)" : "+v"(k[0]), "+v"(k[1]), "+v"(k[2]), "+v"(k[3]));
+    else if (N == 4) asm volatile("s_waitcnt lgkmcnt(4)" : "+v"(k[0]), "+v"(k[1]), "+v"(k[2]), "+v"(k[3]));
+    else asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(k[0]), "+v"(k[1]), "+v"(k[2]), "+v"(k[3]));
+}
 // The transposing reads are issued in two groups of four (first vfr[0..3], then vfr[4..7]). LDS operations complete in order, so
 // once at most four are outstanding the first group has landed whatever else the compiler has put in between.
 __device__ __forceinline__ void lds_wait_first4(uint2 (&a)[8]) {
@@ -99,7 +125,18 @@ __device__ __forceinline__ void lds_wait_last4(uint2 (&a)[8]) {
 // direct global->LDS path). Without it q and k are taken as they are (already normalised by the QKV GEMM epilogue).
 template <bool NORM>
 __global__ void __launch_bounds__(NW * 64, 2) flash_attn_bf16_kernel(const AttnSets sets, float q_scale /* log2(e)/sqrt(64) */, float eps) {
-    __shared__ __attribute__((aligned(1024))) char smem[SMEM_BYTES];
+    constexpr int PF = prefetch_tiles(NORM);
+    __shared__ __attribute__((aligned(1024))) char smem[smem_bytes(NORM)];
+    // The barrier in the middle of a tile, which publishes tile t+1 and retires the stage of tile t-1. In front of it a thread's own
+    // requests for tile t+1 must have landed -- every thread requests four 16-byte chunks per tile, so that is "all but the newest
+    // 4 (PF - 1)" -- and its LDS accesses must be done. A bare barrier between compiler fences: __syncthreads() would wait for
+    // every load in flight, the tiles requested further ahead included.
+    auto tile_barrier = [&]() {
+        __builtin_amdgcn_s_waitcnt(((4 * (PF - 1)) & 15) | (7 << 4) | (0 << 8));  // vmcnt(4 (PF - 1)), lgkmcnt(0)
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+    };
     const int which = (blockIdx.x >= (unsigned)sets.end[0]) + (blockIdx.x >= (unsigned)sets.end[1]);  // uniform
     const SegDev& s = sets.set[which];
     const int wg_first = which ? sets.end[which - 1] : 0;
@@ -196,10 +233,13 @@ __global__ void __launch_bounds__(NW * 64, 2) flash_attn_bf16_kernel(const AttnS
     const bf16_t* vp[2];
     // advance() moves the four row pointers to the tile that starts at key t0 (branches; kept out of the pipeline steps),
     // fetch_tile() issues the loads through them (straight-line; interleaved with a step's matrix instructions)
+    // (the two strides are read once, here: inside advance() the set's row stride, a kernel argument selected by `which`, was a
+    // scalar memory load and a wait for it in the middle of every tile)
+    const long long tile_step0 = (long long)BKV * s.ld_qkv[0], tile_step1 = (long long)BKV * s.ld_qkv[1];
     auto advance = [&](int t0) {
         const bool in0 = (t0 >= kv0 + BKV) && (t0 + BKV <= T0), in1 = (t0 - BKV >= max(T0, kv0)) && (t0 + BKV <= T);
         if (in0 || in1) {
-            const long long step = (long long)BKV * s.ld_qkv[in1 ? 1 : 0];
+            const long long step = in1 ? tile_step1 : tile_step0;
 #pragma unroll
             for (int i = 0; i < 2; i++) {
                 kp[i] += step;
@@ -311,15 +351,10 @@ __global__ void __launch_bounds__(NW * 64, 2) flash_attn_bf16_kernel(const AttnS
         }
         aux.u = make_uint4(0u, 0u, 0u, 0u);
     };
-    auto scores = [&](auto fast, int qb, int key_base) {
-        constexpr bool FAST = decltype(fast)::value;
-        if (FAST) {
-            sacc[qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[0], qf[qb][0].v, zero, 0, 0, 0);
-        } else {
-            aux.u.x = (key_base >= first_masked) ? 0x3f803f80u : 0x00003f80u;
-            sacc[qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(aux.v, negm_f[qb].v, zero, 0, 0, 0);
-            sacc[qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[0], qf[qb][0].v, sacc[qb], 0, 0, 0);
-        }
+    auto scores = [&](int qb, int key_base) {
+        aux.u.x = (key_base >= first_masked) ? 0x3f803f80u : 0x00003f80u;
+        sacc[qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(aux.v, negm_f[qb].v, zero, 0, 0, 0);
+        sacc[qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[0], qf[qb][0].v, sacc[qb], 0, 0, 0);
 #pragma unroll
         for (int ks = 1; ks < 4; ks++) sacc[qb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[ks], qf[qb][ks].v, sacc[qb], 0, 0, 0);
     };
@@ -400,81 +435,177 @@ __global__ void __launch_bounds__(NW * 64, 2) flash_attn_bf16_kernel(const AttnS
         }
         l_run[qb] += inc;
     };
-    // one matrix instruction, then a few vector instructions, nine times: the mix of one pipeline step of the general path.
-    // (Fast tiles go without: every such pattern tried there -- 1:2 to 1:5, pairs, with the transcendental class named -- measured
-    // 7 % slower than what the compiler's own scheduler does with the shorter step.)
-    auto interleave = [&](auto fast) {
-        if (decltype(fast)::value) return;
+    // one matrix instruction, then a few vector instructions, nine times: the mix of one pipeline step of the general path
+    auto interleave = [&]() {
 #pragma unroll
         for (int i = 0; i < 9; i++) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
             __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
         }
     };
-    // A fast tile keeps the reference at zero and only adds up; whether that was safe is looked at once, behind the last of them.
-    auto account = [&](auto fast, int qb, float inc, bool force) {
-        if (decltype(fast)::value) {
-            l_run[qb] += inc;
-        } else {
-            settle(qb, inc, force);
-        }
-    };
 
     // Stages of tiles t, t+1, t+2
-    int st_cur, st_nxt, st_ld;
-    // One tile of the pipeline: four steps. FAST tiles are those in which no key is masked and the reference is known to be zero.
-    auto tile = [&](auto fast, int t) {
+    int st_cur, st_nxt, st_nx2, st_ld;
+    auto rotate_stages = [&]() {
+        const int tmp = st_cur;
+        st_cur = st_nxt;
+        if (PF == 2) {
+            st_nxt = st_nx2;
+            st_nx2 = st_ld;
+        } else {
+            st_nxt = st_ld;
+        }
+        st_ld = tmp;
+    };
+    // One tile of the pipeline on the general path (any key may be masked, the reference may move): four steps.
+    auto tile = [&](int t) {
         float inc;
         // ---- step (t, 0, 0): PV of (t-1,1,1), each half followed by the fetch of V of key half 0 into the registers it
         //      frees; scores of (t,0,1); then fetch K of half 1 ----
         pv(1, 0);
         load_v(st_cur, 0, 0);
-        scores(fast, 1, kv0 + t * BKV);
+        scores(1, kv0 + t * BKV);
         load_k(st_cur, 1);
         inc = probs(0);
         pv(1, 1);
         load_v(st_cur, 0, 1);
-        interleave(fast);
-        account(fast, 0, inc, t == 0);
+        interleave();
+        settle(0, inc, t == 0);
         // ---- step (t, 0, 1): PV of (t,0,0); scores of (t,1,0) ----
         lds_wait_first4(vfr);
         pv(0, 0);
-        scores(fast, 0, kv0 + t * BKV + 32);
+        scores(0, kv0 + t * BKV + 32);
         inc = probs(1);
         lds_wait_last4(vfr);
         pv(0, 1);
-        interleave(fast);
-        account(fast, 1, inc, t == 0);
+        interleave();
+        settle(1, inc, t == 0);
         // ---- step (t, 1, 0): tile t+1 becomes visible and the loads of tile t+2 set off (past the end: the last tile once
         //      more, into a stage nobody reads again); PV of (t,0,1) and fetch of V of key half 1; scores of (t,1,1); then
         //      fetch K of half 0 of tile t+1 (past the last tile: stale LDS, feeding scores that are never used) ----
         if (NORM && t + 1 < nt) store_k_normed(kv0 + (t + 1) * BKV, st_nxt);
-        __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8));  // vmcnt(0): this thread's loads of tile t+1 have landed
-        __syncthreads();  // (also in the last tile: the stage the redundant loads go to must not be in use by a slower wavefront)
-        if (t + 2 < nt) advance(kv0 + (t + 2) * BKV);
+        tile_barrier();  // (also in the last tile: the stage the redundant loads go to must not be in use by a slower wavefront)
+        if (t + PF + 1 < nt) advance(kv0 + (t + PF + 1) * BKV);
         fetch_tile(st_ld);
         pv(1, 0);
         load_v(st_cur, 1, 0);
-        scores(fast, 1, kv0 + t * BKV + 32);
+        scores(1, kv0 + t * BKV + 32);
         load_k(st_nxt, 0);
         inc = probs(0);
         pv(1, 1);
         load_v(st_cur, 1, 1);
-        interleave(fast);
-        account(fast, 0, inc, false);
+        interleave();
+        settle(0, inc, false);
         // ---- step (t, 1, 1): PV of (t,1,0); scores of (t+1,0,0) ----
         lds_wait_first4(vfr);
         pv(0, 0);
-        scores(fast, 0, kv0 + t * BKV + BKV);
+        scores(0, kv0 + t * BKV + BKV);
         inc = probs(1);
         lds_wait_last4(vfr);
         pv(0, 1);
-        interleave(fast);
-        account(fast, 1, inc, false);
-        const int tmp = st_cur;
-        st_cur = st_nxt;
-        st_nxt = st_ld;
-        st_ld = tmp;
+        interleave();
+        settle(1, inc, false);
+        rotate_stages();
+    };
+
+    // ---- a fast tile with the instruction order written out. Left to itself the compiler bunches the matrix instructions of a
+    //      step (six in a row behind the barrier, thirty vector instructions in a row elsewhere). Here every step is eight slices of
+    //      {one matrix instruction; an eighth of the step's vector work: 2 exp2, 1 conversion, 2 additions}, and nothing moves across
+    //      a slice boundary. Order inside a step: the four score products first (the K fragments are then free: the next key half
+    //      is fetched right behind them and has four slices to arrive), then PV of the first key quarter, then of the second, each
+    //      followed in even steps by the fetch of the next V fragments into the registers just read. All LDS reads of these
+    //      tiles are issued from assembly and waited for by count; exp2 of a pair of scores is issued one slice ahead of its
+    //      conversion. Measured against the compiler's order on one device, 1536 workgroups of 64 tiles: 6 % faster with all-zero
+    //      operands, 1.7 % with N(0,1) operands, where the power limit and not the instruction stream sets the pace. (Also tried
+    //      on this basis: the row sums as two more matrix instructions per unit, ONES . P^T, instead of 16 additions: 7.5 % faster
+    //      on zeros, 3 % slower on N(0,1) operands; the requests for the next tile spread over a step: slower.) ----
+    auto fast_step = [&](auto qb_tag, auto loads_tag, auto vkb_tag, int v_stage, auto kkb_tag, int k_stage) {
+        constexpr int QB = decltype(qb_tag)::value, PQ = QB ^ 1;     // probabilities of query block QB; scores and PV of the other one
+        constexpr bool LOADS = decltype(loads_tag)::value;          // even steps fetch K of the next key half and V of this one
+        constexpr int VKB = decltype(vkb_tag)::value, KKB = decltype(kkb_tag)::value;
+        // The vector instructions are written as assembly statements, which the compiler keeps in the order given (as plain
+        // arithmetic it sinks the conversions to where their results are needed, a step later). What the compiler's hazard
+        // handling cannot see through them holds by construction: a score block is read here four or more slices behind the last
+        // matrix instruction that wrote it, the operands packed here are read by matrix instructions of the next step, and no
+        // exp2 result is used by the instruction right behind it.
+        float e[2][2];
+        uint32_t w[8];
+        auto exps = [&](int c) {
+            asm volatile("v_exp_f32 %0, %1" : "=v"(e[c & 1][0]) : "v"(sacc[QB][2 * c]));
+            asm volatile("v_exp_f32 %0, %1" : "=v"(e[c & 1][1]) : "v"(sacc[QB][2 * c + 1]));
+        };
+        auto convert = [&](int c) { asm volatile("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(w[c]) : "v"(e[c & 1][0]), "v"(e[c & 1][1])); };
+        // Sum of pair c and its two partial sums: the same pairs and the same partial sums as pack_probs. A dependent vector
+        // instruction right behind its producer costs a wait state, so the sum of a pair joins its partial sum a slice later.
+        float pair[2], ls[2];
+        auto add_pair = [&](int c) {
+            if (c < 2) asm volatile("v_add_f32 %0, %1, %2" : "=v"(ls[c & 1]) : "v"(e[c & 1][0]), "v"(e[c & 1][1]));
+            else asm volatile("v_add_f32 %0, %1, %2" : "=v"(pair[c & 1]) : "v"(e[c & 1][0]), "v"(e[c & 1][1]));
+        };
+        auto join = [&](int c) {
+            if (c >= 2) asm volatile("v_add_f32 %0, %0, %1" : "+v"(ls[c & 1]) : "v"(pair[c & 1]));
+        };
+        if (!LOADS) lds_wait_k<8>(kf);  // the K fragments fetched in the step before (eight V reads may still be on their way)
+        // matrix instructions of the step: 0-3 scores; 4, 5 PV of key quarter 0; 6, 7 PV of quarter 1
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            if (i < 4) {
+                sacc[PQ] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[i], qf[PQ][i].v, i == 0 ? zero : sacc[PQ], 0, 0, 0);
+            } else {
+                const int j = (i - 4) >> 1, db = (i - 4) & 1;
+                if (!LOADS && i == 4) lds_wait_first4(vfr);
+                if (!LOADS && i == 6) lds_wait_last4(vfr);
+                Frag vf;
+                vf.u = make_uint4(vfr[(j * 2 + db) * 2].x, vfr[(j * 2 + db) * 2].y, vfr[(j * 2 + db) * 2 + 1].x, vfr[(j * 2 + db) * 2 + 1].y);
+                oacc[db][PQ] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf.v, pf[PQ][j].v, oacc[db][PQ], 0, 0, 0);
+            }
+            if (LOADS && i == 3) {
+#pragma unroll
+                for (int ks = 0; ks < 4; ks++) kf[ks] = lds_read_b128(smem_addr + k_stage + koff[ks], KKB * 32 * 128);
+            }
+            if (LOADS && (i == 5 || i == 7)) {
+                const int j = (i - 4) >> 1;
+#pragma unroll
+                for (int db = 0; db < 2; db++)
+#pragma unroll
+                    for (int hi = 0; hi < 2; hi++)
+                        vfr[(j * 2 + db) * 2 + hi] = lds_read_tr16_b64(smem_addr + v_stage + voff[db], (VKB * 32 + 16 * j + 8 * hi) * 128);
+            }
+            if (i == 0) exps(0);
+            if (i > 0) convert(i - 1);
+            if (i > 1) join(i - 2);
+            if (i > 0) add_pair(i - 1);
+            if (i < 7) exps(i + 1);
+            if (i == 7) {  // the tail of the step's vector work: the last pair and the row-sum update (a short dependent chain)
+                convert(7);
+                join(6);
+                add_pair(7);
+                asm volatile("v_nop");
+                join(7);
+                float both;
+                asm volatile("v_add_f32 %0, %1, %2" : "=v"(both) : "v"(ls[0]), "v"(ls[1]));
+                asm volatile("v_nop");
+                asm volatile("v_add_f32 %0, %0, %1" : "+v"(l_run[QB]) : "v"(both));
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        pf[QB][0].u = make_uint4(w[0], w[1], w[2], w[3]);
+        pf[QB][1].u = make_uint4(w[4], w[5], w[6], w[7]);
+    };
+    auto fast_tile = [&](int t) {
+        const std::integral_constant<int, 0> I0;
+        const std::integral_constant<int, 1> I1;
+        const std::integral_constant<bool, true> YES;
+        const std::integral_constant<bool, false> NO;
+        fast_step(I0, YES, I0, st_cur, I1, st_cur);  // (t,0,0): V of key half 0, K of key half 1
+        fast_step(I1, NO, I0, 0, I0, 0);             // (t,0,1)
+        tile_barrier();
+        if (t + PF + 1 < nt) advance(kv0 + (t + PF + 1) * BKV);
+        fetch_tile(st_ld);
+        __builtin_amdgcn_sched_barrier(0);
+        fast_step(I0, YES, I1, st_cur, I0, st_nxt);  // (t,1,0): V of key half 1, K of key half 0 of tile t+1
+        fast_step(I1, NO, I0, 0, I0, 0);             // (t,1,1)
+        rotate_stages();
     };
 
     // Fast tiles: the leading tiles whose units, and the unit whose scores the last of them issues (the first of the next tile), lie
@@ -490,8 +621,6 @@ __global__ void __launch_bounds__(NW * 64, 2) flash_attn_bf16_kernel(const AttnS
     constexpr float L_TINY = 5.421010862427522e-20f /* 2^-64 */, L_HUGE = 1099511627776.0f /* 2^40 */;
     int n_fast = (kv0 + nt * BKV <= T) ? nt : min(nt, (T - kv0 - 32) / BKV);
     if (NORM || n_fast < 4) n_fast = 0;
-    const std::integral_constant<bool, true> FAST_TILE;
-    const std::integral_constant<bool, false> ANY_TILE;
 
     for (;;) {
         reset();
@@ -504,18 +633,31 @@ __global__ void __launch_bounds__(NW * 64, 2) flash_attn_bf16_kernel(const AttnS
         asm volatile("" : "+s"(first_key));
         advance(first_key);
         fetch_tile(0);
-        if (NORM) store_k_normed(kv0, 0);
-        if (nt > 1) {
-            advance(first_key + BKV);
-            fetch_tile(STAGE_BYTES);
-            __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8) | 4);  // vmcnt(4): all but the four loads of tile 1
+        if (PF == 1) {
+            if (NORM) store_k_normed(kv0, 0);
+            if (nt > 1) {
+                advance(first_key + BKV);
+                fetch_tile(STAGE_BYTES);
+                __builtin_amdgcn_s_waitcnt((7 << 4) | (0 << 8) | 4);  // vmcnt(4): all but the four loads of tile 1; lgkmcnt(0)
+            } else {
+                __builtin_amdgcn_s_waitcnt((7 << 4) | (0 << 8));
+            }
+            st_cur = 0, st_nxt = STAGE_BYTES, st_nx2 = 0, st_ld = 2 * STAGE_BYTES;
         } else {
-            __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8));
+            // two more tiles on their way (a sequence shorter than that: its last tile once more, so that the count of requests in
+            // flight is the same for every length and "tile t+1 has landed" is a fixed count in the loop)
+            if (nt > 1) advance(first_key + BKV);
+            fetch_tile(STAGE_BYTES);
+            if (nt > 2) advance(first_key + 2 * BKV);
+            fetch_tile(2 * STAGE_BYTES);
+            __builtin_amdgcn_s_waitcnt((7 << 4) | (0 << 8) | 8);  // vmcnt(8): all but the eight loads of tiles 1 and 2; lgkmcnt(0)
+            st_cur = 0, st_nxt = STAGE_BYTES, st_nx2 = 2 * STAGE_BYTES, st_ld = 3 * STAGE_BYTES;
         }
-        __syncthreads();
+        asm volatile("" ::: "memory");  // (a bare barrier: __syncthreads() would wait for the tiles requested ahead as well)
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
         load_k(0, 0);
-        scores(ANY_TILE, 0, kv0);
-        st_cur = 0, st_nxt = STAGE_BYTES, st_ld = 2 * STAGE_BYTES;
+        scores(0, kv0);
 
         // verdict on the fast tiles so far, the same for every wavefront of the workgroup: flags raised in front of a barrier, read behind it
         auto unsafe = [&]() -> bool {
@@ -525,11 +667,11 @@ __global__ void __launch_bounds__(NW * 64, 2) flash_attn_bf16_kernel(const AttnS
             __syncthreads();
             return __builtin_amdgcn_readfirstlane(*flag) != 0;
         };
-        for (int t = 0; t < n_fast; t++) tile(FAST_TILE, t);
+        for (int t = 0; t < n_fast; t++) fast_tile(t);
         const bool redo = n_fast > 0 && unsafe();
         if (!redo) {
             if (n_fast > 0) zero_reference();
-            for (int t = n_fast; t < nt; t++) tile(ANY_TILE, t);
+            for (int t = n_fast; t < nt; t++) tile(t);
             break;
         }
         // start again without fast tiles, once every wavefront is done with the LDS stages and no load into them is in flight
