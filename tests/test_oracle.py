@@ -205,6 +205,58 @@ def block64(y, c, x, P, NH, dual, qk, disc):
     return c, x
 
 
+# ---------------------------------------------------------------- float64 forward written from the op list (modules.cpp:1660-1752)
+def dit64(pooled, captions, latent, timesteps, P, cfg):
+    f = lambda n: P[n].astype(np.float64)  # noqa: E731
+    silu = lambda a: a / (1 + np.exp(-a))  # noqa: E731
+    pooled, captions, latent, t = (a.astype(np.float64) for a in (pooled, captions, latent, timesteps))
+    B, Cin, H, W = latent.shape
+    C, p = cfg.emb_dim, cfg.patch_size
+    Hp, Wp = H // p, W // p
+    # conditioning vector: [cos | sin] of t * 10000^(-i/128), two MLPs, sum, silu (modules.cpp:920-944, 1663-1675)
+    freq = np.exp(-np.log(10000.0) * 2 * np.arange(128) / 256)
+    temb = np.concatenate([np.cos(t[:, None] * freq), np.sin(t[:, None] * freq)], 1)
+    mlp = lambda a, n: silu(a @ f(n + ".0.weight") + f(n + ".0.bias")) @ f(n + ".2.weight") + f(n + ".2.bias")  # noqa: E731
+    y = silu(mlp(temb, "timestep_mlp") + mlp(pooled, "pooled_mlp"))
+    c = captions @ f("captions_linear.weight") + f("captions_linear.bias")
+    # patch embedding: p x p / stride p convolution, tokens in row-major patch order (modules.cpp:1037-1062, 1093-1117)
+    patches = latent.reshape(B, Cin, Hp, p, Wp, p).transpose(0, 2, 4, 1, 3, 5).reshape(B, Hp * Wp, Cin * p * p)
+    x = patches @ f("to_patch.conv.weight").reshape(C, Cin * p * p).T + f("to_patch.conv.bias")
+    # position table (modules.cpp:946-995): entry [a][b] of the max x max table uses a for the "width" angle and b for the "height"
+    # angle, [sin h | cos h | sin w | cos w]; the centre crop reads it as [row][col]
+    mx, base = cfg.pos_embed_max_size, cfg.base_height // p
+    fr = 1.0 / np.power(10000.0, 4.0 * np.arange(C // 4) / C)
+    oh, ow = (mx - Hp) // 2, (mx - Wp) // 2
+    pw = (np.arange(Hp) + oh)[:, None] * base / mx      # rows of the crop index the table's first ("width") axis
+    ph = (np.arange(Wp) + ow)[:, None] * base / mx
+    e_h = np.concatenate([np.sin(ph * fr), np.cos(ph * fr)], 1)   # (Wp, C/2)
+    e_w = np.concatenate([np.sin(pw * fr), np.cos(pw * fr)], 1)   # (Hp, C/2)
+    pos = np.concatenate([np.broadcast_to(e_h[None], (Hp, Wp, C // 2)), np.broadcast_to(e_w[:, None], (Hp, Wp, C // 2))], 2).reshape(Hp * Wp, C)
+    x = x + pos.astype(np.float32).astype(np.float64)             # (the reference stores the table as float)
+    for l in range(cfg.num_layers):
+        pre = f"transformer.{l}."
+        Pl = {n[len(pre):]: v for n, v in P.items() if n.startswith(pre)}
+        c, x = block64(y, c, x, Pl, cfg.attn_heads, l in cfg.dual_attention_layers, cfg.use_qk_norm, l == cfg.num_layers - 1)
+    m = x.mean(-1, keepdims=True)
+    xh = (x - m) / np.sqrt(((x - m) ** 2).mean(-1, keepdims=True) + 1e-5)
+    scale, shift = np.split(y @ f("ada_ln_out.linear.weight") + f("ada_ln_out.linear.bias"), 2, -1)   # chunk 0 = scale, chunk 1 = shift
+    tok = (xh * (1 + scale[:, None]) + shift[:, None]) @ f("linear_out.weight") + f("linear_out.bias")
+    # tokens -> pixels: channel index of a token is (ph * p + pw) * C_in + ch (modules.cpp:1730-1752)
+    return tok.reshape(B, Hp, Wp, p, p, Cin).transpose(0, 5, 1, 3, 2, 4).reshape(B, Cin, H, W)
+
+
+@pytest.mark.parametrize("name", list(cases.DIT_CASES))
+def test_float64_forward_written_from_the_op_list_vs_oracle_and_golden(name):
+    """Pins dit64 (used by the GPU tests at sizes the CPU oracle cannot reach in a test run) to the oracle and to the compiled
+    reference's output, conventions included: [cos|sin] order, position-table axes and crop, scale/shift swap, un-patchify order."""
+    k = cases.dit_case(name)
+    out64 = dit64(k["pooled"], k["captions"], k["latent"], k["timesteps"], k["params"], k["cfg"])
+    out = ol.orc_dit_forward(k["pooled"], k["captions"], k["latent"], k["timesteps"], k["params"], k["cfg"])
+    scale = max(1.0, np.abs(out64).max())
+    assert np.abs(out - out64).max() < 2e-4 * scale
+    assert np.abs(GOLDEN[name + ".out"] - out64).max() < 2e-4 * scale
+
+
 @pytest.mark.parametrize("name", list(cases.BLOCK_CASES))
 def test_block_vs_float64_numpy_and_golden(name):
     k = cases.block_case(name)
