@@ -148,16 +148,17 @@ def test_block_fp32_baseline_config1_vs_float64(dual):
     assert max_abs(x, x64) <= F32_TOL and max_abs(c, c64) <= F32_TOL
 
 
-@pytest.mark.parametrize("dual,discard", [(True, False), (False, True)])
-def test_block_bf16_at_512px_token_counts_vs_float64(dual, discard):
-    """The block at the token counts of BASELINE config 3 (batch 2, 1024 image + 154 text tokens, width 1536), with weights of standard
-    deviation 0.05 so that the modulation vectors and gates are of order 2 and every branch weighs heavily in the result: the bf16 path
-    against the float64 statement of the block directly (not through the fp32 GPU path), and the fp32 path against the same."""
+@pytest.mark.parametrize("dual,discard,B,Tx", [(True, False, 2, 1024), (False, True, 2, 1024), (True, False, 1, 4096)])
+def test_block_bf16_at_512px_and_1024px_token_counts_vs_float64(dual, discard, B, Tx):
+    """The block at the token counts of BASELINE config 3 (batch 2, 1024 image + 154 text tokens, width 1536) and, one batch element, of
+    the headline shape (4096 + 154), with weights of standard deviation 0.05 so that the modulation vectors and gates are of order 2
+    and every branch weighs heavily in the result: the bf16 path against the float64 statement of the block directly (not through
+    the fp32 GPU path), and the fp32 path against the same."""
     rng = np.random.Generator(np.random.Philox(71))
     C, NH = 1536, 24
     params = synthetic_params_numpy(block_param_shapes(C, 4, dual, True, discard, C // NH), 72, 0.05, 0.05)
-    k = dict(y=rng.standard_normal((2, C), dtype=np.float32), c=rng.standard_normal((2, 154, C), dtype=np.float32),
-             x=rng.standard_normal((2, 1024, C), dtype=np.float32), params=params, NH=NH, mlp_expand=4, use_dual=dual, use_qk_norm=True,
+    k = dict(y=rng.standard_normal((B, C), dtype=np.float32), c=rng.standard_normal((B, 154, C), dtype=np.float32),
+             x=rng.standard_normal((B, Tx, C), dtype=np.float32), params=params, NH=NH, mlp_expand=4, use_dual=dual, use_qk_norm=True,
              discard_context=discard)
     c64, x64 = block64(k["y"], k["c"], k["x"], k["params"], NH, dual, True, discard)
     assert rel_l2(x64 - k["x"], k["x"]) > 1.0                     # the update is larger than what it is added to
