@@ -162,14 +162,14 @@ def test_gemm_bf16_result_does_not_depend_on_tile_shape(Mr, N, K, epi):
     bias = torch.randn(N, device="cuda", generator=g)
     outs = []
     try:
-        for tile in (128, 256, 0):
+        for tile in (128, 256, 0, 192):
             L.call("sd3_gemm_bf16_force_tile", tile)
             out = torch.zeros((Mr, N), device="cuda", dtype=torch.bfloat16)
             L.call("sd3_gemm_bf16", A.data_ptr(), Wp.data_ptr(), bias.data_ptr(), out.data_ptr(), Mr, N, K, epi, None)
             outs.append(out)
     finally:
         L.call("sd3_gemm_bf16_force_tile", 0)
-    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
+    assert all(torch.equal(outs[0], o) for o in outs[1:])
     with pytest.raises(L.Sd3Error):
         L.call("sd3_gemm_bf16_force_tile", 64)
 
