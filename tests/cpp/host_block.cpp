@@ -86,6 +86,35 @@ int main(int argc, char** argv) {
     };
     const bool ok = dump(c, (size_t)B * Tc * C) && dump(x, mx * C) && dump(lin, mx * C) && dump(mlp_out, mx * C);
     std::fclose(o);
-    sd3_ctx_destroy(sd3::modules_ctx());
-    return ok ? 0 : 74;
+    if (!ok) return 74;
+
+    // Stream lifetime: the same block twice more, each time on a stream that this program creates before the call and destroys
+    // after it. When the second call hands the context its new stream the previous one no longer exists, and when the context is
+    // destroyed neither does: the library must order its work without touching a dead stream's handle, and give the same bits.
+    std::vector<float> first(mx * C), again(mx * C);
+    HIP_OK(hipMemcpy(first.data(), x, mx * C * sizeof(float), hipMemcpyDeviceToHost));
+    for (int round = 0; round < 2; round++) {
+        hipStream_t s = nullptr;
+        HIP_OK(hipStreamCreate(&s));
+        sd3::modules_stream() = s;
+        HIP_OK(hipMemcpyAsync(c, host[1].data(), host[1].size() * sizeof(float), hipMemcpyHostToDevice, s));
+        HIP_OK(hipMemcpyAsync(x, host[2].data(), host[2].size() * sizeof(float), hipMemcpyHostToDevice, s));
+        try {
+            dit_block(y, c, x, w[0], w[1], w[2], w[3], w[4], w[5], w[6], w[7], w[8], w[9], w[10], w[11], w[12], w[13], w[14], w[15], w[16], w[17],
+                      w[18], w[19], w[20], w[21], w[22], w[23], w[24], w[25], w[26], w[27], w[28], w[29], none, none, none, none, none, none, none,
+                      none, none, none, none, none, none, none, none, none, B, Tc, Tx, C, NH, E, dual, qk, discard);
+        } catch (const std::exception& e) {
+            std::fprintf(stderr, "stream round %d: %s\n", round, e.what());
+            return 1;
+        }
+        HIP_OK(hipMemcpyAsync(again.data(), x, mx * C * sizeof(float), hipMemcpyDeviceToHost, s));
+        HIP_OK(hipStreamSynchronize(s));
+        HIP_OK(hipStreamDestroy(s));
+        if (std::memcmp(first.data(), again.data(), mx * C * sizeof(float)) != 0) {
+            std::fprintf(stderr, "stream round %d: result differs from the first call\n", round);
+            return 75;
+        }
+    }
+    if (sd3_ctx_destroy(sd3::modules_ctx()) != SD3_OK) return 76;  // (its last stream is gone by now)
+    return 0;
 }

@@ -44,7 +44,9 @@ def test_cpp_program_calls_dit_block_linear_and_mlp_with_the_reference_argument_
     case, out = str(tmp_path / "case.bin"), str(tmp_path / "out.bin")
     _write_case(case, k)
     r = subprocess.run([exe, case, out] + (["bf16"] if mode == "bf16" else []), capture_output=True, text=True, timeout=120)
-    assert r.returncode == 0, r.stderr
+    # 0 also says that the program's two further calls, each on a stream created before and destroyed after it, gave the bits of the
+    # first call (75 otherwise) and that the context could be destroyed after its last stream was (76 otherwise)
+    assert r.returncode == 0, (r.returncode, r.stderr)
     B, Tc, C = k["c"].shape
     Tx, E = k["x"].shape[1], k["mlp_expand"]
     got = np.fromfile(out, np.float32)
