@@ -37,8 +37,34 @@ def _up(t):
     return t.detach().to(device=_DEV, dtype=torch.float32).contiguous()
 
 
+_uploaded = {}  # name -> (tensor of the caller, its version counter, the device copy)
+
+
 def _params_up(params):
-    return {k: _up(v) for k, v in params.items()}
+    """Device copies of a parameter map. The reference's entry points receive the whole map on every call; a tensor that is the same
+    object (or the same memory) with the same torch version counter as in the previous call keeps its device copy, so a sampling
+    loop uploads the weights once and the context behind `Dit_block` / `DiT` keeps what it derived from them. Tensors that are on
+    the GPU already, in float32 and contiguous, are passed through. `release()` drops the copies."""
+    out = {}
+    for name, t in params.items():
+        old = _uploaded.get(name)
+        if old is not None and (old[0] is t or (old[0].data_ptr() == t.data_ptr() and old[0].shape == t.shape and old[0].dtype == t.dtype)) \
+                and old[1] == t._version:
+            out[name] = old[2]
+            continue
+        d = _up(t)
+        _uploaded[name] = (t, t._version, d)
+        out[name] = d
+    for name in [n for n in _uploaded if n not in params]:
+        del _uploaded[name]
+    return out
+
+
+def release():
+    """Frees what the module keeps between calls: the device copies of the last parameter map and the contexts behind `Dit_block` /
+    `DiT` (their bf16 weight copies and workspaces)."""
+    _uploaded.clear()
+    _M.release_shared_contexts()
 
 
 def _host_op(fn):
@@ -75,27 +101,28 @@ def positional_embedding(emb_dim, height, width, base_size):
 
 
 def Dit_block(temp_embeddings, context_embeddings, latent_vector, params, B, Tc, Tx, emb_dim, attn_heads, mlp_expand, use_dual_attention, use_qk_norm,
-              discard_context):
-    """modules.cpp:1508 DiT_block_forward on host tensors: context_embeddings and latent_vector are updated in place and returned."""
+              discard_context, precision=None):
+    """modules.cpp:1508 DiT_block_forward on host tensors: context_embeddings and latent_vector are updated in place and returned.
+    `precision` (not in the reference's list) overrides the module-level PRECISION for this call."""
     y, c, x = _up(temp_embeddings), _up(context_embeddings), _up(latent_vector)
     c, x = _M.Dit_block(y, c, x, _params_up(params), B, Tc, Tx, emb_dim, attn_heads, mlp_expand, use_dual_attention, use_qk_norm, discard_context,
-                        precision=PRECISION)
+                        precision=precision or PRECISION)
     context_embeddings.copy_(c.to(context_embeddings.device))
     latent_vector.copy_(x.to(latent_vector.device))
     return [context_embeddings, latent_vector]
 
 
 def DiT_block_cuda(temp_embeddings, context_embeddings, latent_vector, params, B, Tc, Tx, emb_dim, attn_heads, mlp_expand, use_dual_attention,
-                   use_qk_norm, discard_context):
+                   use_qk_norm, discard_context, precision=None):
     """modules.cpp:1783 DiT_block_forward_cuda: device tensors, updated in place and returned."""
     return _M.Dit_block(temp_embeddings, context_embeddings, latent_vector, params, B, Tc, Tx, emb_dim, attn_heads, mlp_expand, use_dual_attention,
-                        use_qk_norm, discard_context, precision=PRECISION)
+                        use_qk_norm, discard_context, precision=precision or PRECISION)
 
 
 def DiT(pooled_captions, captions, latent_vector, timesteps, params, num_layers, dual_attention_layers, pooled_dim, captions_dim, C_in, emb_dim, attn_heads,
-        mlp_expand, patch_size, pos_embed_max_size, base_height, use_qk_norm):
+        mlp_expand, patch_size, pos_embed_max_size, base_height, use_qk_norm, precision=None):
     """modules.cpp:1605 DiT_forward on host (or device) tensors: returns a new (B, C_in, H, W) tensor on the latent's device."""
     out = _M.DiT(_up(pooled_captions), _up(captions), _up(latent_vector), _up(timesteps), _params_up(params), num_layers, dual_attention_layers,
                  pooled_dim, captions_dim, C_in, emb_dim, attn_heads, mlp_expand, patch_size, pos_embed_max_size, base_height, use_qk_norm,
-                 precision=PRECISION)
+                 precision=precision or PRECISION)
     return out.to(latent_vector.device)

@@ -67,6 +67,41 @@ def test_module_level_precision_switch_reaches_the_bf16_path():
     assert 1e-6 < rel_l2(x.numpy(), gold) <= 1e-2
 
 
+def test_host_parameter_map_is_uploaded_once_and_follows_in_place_changes():
+    """The reference's signatures hand the host parameter map to every call. A second call with the same map re-uses the device copies
+    (and, in bf16, the weight copies derived from them); a weight changed in place is uploaded again and the result follows it; the
+    per-call `precision` keyword overrides the module-level switch."""
+    from gpu_util import rel_l2
+    k = cases.block_case("block_dual_hs64")
+    (B, Tc, C), Tx = k["c"].shape, k["x"].shape[1]
+    params = {n: torch.from_numpy(v.copy()) for n, v in k["params"].items()}
+    args = (B, Tc, Tx, C, k["NH"], k["mlp_expand"], k["use_dual"], k["use_qk_norm"], k["discard_context"])
+
+    def run(precision):
+        y, c, x = torch.from_numpy(k["y"].copy()), torch.from_numpy(k["c"].copy()), torch.from_numpy(k["x"].copy())
+        F.Dit_block(y, c, x, params, *args, precision=precision)
+        return x
+
+    F.release()
+    x1 = run("bf16")
+    copies = {n: v[2].data_ptr() for n, v in F._uploaded.items()}
+    ctx = F._M.shared_context("cuda")
+    built = ctx.copies_built()
+    assert set(copies) == set(params) and built > 0
+    x2 = run("bf16")
+    assert {n: v[2].data_ptr() for n, v in F._uploaded.items()} == copies and ctx.copies_built() == built
+    assert torch.equal(x1, x2) and 1e-6 < rel_l2(x1.numpy(), GOLDEN["block_dual_hs64.x"]) <= 1e-2
+    assert max_abs(run("fp32").numpy(), GOLDEN["block_dual_hs64.x"]) <= F32_TOL and F.PRECISION == "fp32"
+    name = "latent_mlp.lin2.weight"
+    params[name].mul_(0.5)  # in place: same tensor object, new version counter
+    x3 = run("bf16")
+    assert ctx.copies_built() == built + 1 and not torch.equal(x3, x1)
+    params[name].mul_(2.0)  # (exact: back to the original values)
+    assert torch.equal(run("bf16"), x1)
+    F.release()
+    assert not F._uploaded
+
+
 def test_operator_entry_points_take_host_tensors():
     x = torch.randn(2, 5, 64)
     out = F.layer_norm(x, None, None, 1e-6, False)[0]
