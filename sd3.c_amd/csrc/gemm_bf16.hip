@@ -33,6 +33,13 @@ struct EpiDev {
 // XOR key of an LDS row: rows r..r+7 get 8 different keys (no conflicts on 8-lane / 32-bank groups) and rows r, r+8 get
 // keys that differ in bit 0 (no conflicts on 16-lane / 64-bank groups either).
 __device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 1); }
+// The key for tiles whose fragments are read in the 16x16x32 layout (lane l: row l % 16, chunk 4 * step + l / 16). A 16-byte LDS
+// read is served in four phases of 16 lanes (lanes 0-3, 12-15, 20-23, 24-27; 4-7, 8-11, 16-19, 28-31; the same + 32), so a phase
+// holds rows 0-3 and 12-15 with one chunk index and rows 4-11 with the next: even and odd rows lie in different halves of the 64
+// banks, and row & 6 gives the four even (odd) rows of either group the keys 0, 2, 4, 6 -- with the chunk indices one apart, all
+// eight 16-byte slots of a half. (With swz() that pattern hits every slot twice: the bank-conflict counter read 47 % of the LDS
+// cycles; the 32x32 layout, lane l: row l % 32, is conflict-free with swz() and would not be with this key.)
+__device__ __forceinline__ int swz16(int row) { return row & 6; }
 
 // s_waitcnt vmcnt(n) with the other counters left unconstrained (gfx9 encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[15:14])
 template <int N>
@@ -109,6 +116,8 @@ __device__ __forceinline__ void gemm_tile(const Prob& pr, const int wg, char* sm
     static_assert(BM * 8 % NT == 0 && BN * 8 % NT == 0, "tile rows must divide evenly over the threads");
     static_assert(BM % (WM * 16) == 0 && BN % (WN * 16) == 0 && (BM == 256 || (BM % (WM * 32) == 0 && BN % (WN * 32) == 0)), "wavefront tiles are made of 16x16 (256-row tiles) or 32x32 blocks");
 
+    constexpr bool M16 = (BM == 256) && !FP8;  // 16x16x32 matrix instructions (see below)
+    auto key = [](int row) { return M16 ? swz16(row) : swz(row); };
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: LDS destinations of the direct loads are then scalar
     const int wm = wave / WN, wn = wave % WN;
@@ -122,13 +131,13 @@ __device__ __forceinline__ void gemm_tile(const Prob& pr, const int wg, char* sm
     const long long row_bytes = (long long)K * ESZ;
 #pragma unroll
     for (int i = 0; i < LA; i++) {
-        const int q = i * NT + tid, row = q >> 3, lc = (q & 7) ^ swz(row);
+        const int q = i * NT + tid, row = q >> 3, lc = (q & 7) ^ key(row);
         const int m = min(m_blk + row, M - 1);  // rows beyond M re-read the last row; their results are never stored
         ga[i] = A + (long long)m * row_bytes + lc * 16;
     }
 #pragma unroll
     for (int i = 0; i < LB; i++) {
-        const int q = i * NT + tid, row = q >> 3, lc = (q & 7) ^ swz(row);
+        const int q = i * NT + tid, row = q >> 3, lc = (q & 7) ^ key(row);
         const int n = min(n_blk + row, N - 1);
         gb[i] = Wp + (long long)n * row_bytes + lc * 16;
     }
@@ -145,7 +154,6 @@ __device__ __forceinline__ void gemm_tile(const Prob& pr, const int wg, char* sm
     // the power limit, and measured on random operands the 16x16x32 form sustains 15-24 % more than 32x32x16 at the same nominal
     // rate (half as many accumulator updates per product). 128x128 tiles keep v_mfma_f32_32x32x16_bf16: with four wavefronts per
     // workgroup the finer instruction stream measured 5-15 % slower there. Both forms give bit-identical results.
-    constexpr bool M16 = (BM == 256) && !FP8;
     constexpr int MI = BM / WM / 16, NJ = BN / WN / 16;      // 16x16 blocks per wavefront
     f32x16_t acc[M16 ? 1 : TM][M16 ? 1 : TN];
     f32x4_t acc16[M16 ? MI : 1][M16 ? NJ : 1];
@@ -204,8 +212,8 @@ __device__ __forceinline__ void gemm_tile(const Prob& pr, const int wg, char* sm
     };
     if constexpr (M16) {
         // v_mfma_f32_16x16x32_bf16 operands: lane l holds row (column) l%16 of its block and the 8 consecutive k values 8*(l/16).. of
-        // the 32-deep step: one 16-byte chunk of the row's 128-byte LDS line, chunk (4*step + l/16) ^ swz(row)
-        const int sw = swz(lr);  // (block offsets are multiples of 16 rows, which swz does not see)
+        // the 32-deep step: one 16-byte chunk of the row's 128-byte LDS line, chunk (4*step + l/16) ^ swz16(row)
+        const int sw = swz16(lr);  // (block offsets are multiples of 16 rows, which the key does not see)
         const int a_off = (wm * (BM / WM) + lr) * 128, b_off = A_BYTES + (wn * (BN / WN) + lr) * 128;
         // A fragments: one buffer (the fragment of the next step replaces a[i] as soon as row block i is done), except for the last
         // TAIL row blocks, which have two so that no fragment read is left to issue behind the last matrix instructions of a step
