@@ -54,14 +54,19 @@ def test_dit_bf16_vs_reference_golden():
     assert rel_l2(out, GOLDEN["dit_hs64.out"]) <= BF16_REL_L2
 
 
-@pytest.mark.parametrize("layers,dual,B,side", [(4, (0, 1), 2, 64), (24, tuple(range(13)), 2, 64), (3, (0,), 1, 128)])
+LONG = pytest.mark.skipif(not os.environ.get("SD3_LONG_TESTS"), reason="minutes of float64 numpy on the host: set SD3_LONG_TESTS=1 (and run pytest with -s)")
+
+
+@pytest.mark.parametrize("layers,dual,B,side", [(4, (0, 1), 2, 64), (24, tuple(range(13)), 2, 64), (3, (0,), 1, 128),
+                                                pytest.param(24, tuple(range(13)), 1, 128, marks=LONG)])
 def test_dit_at_512px_and_1024px_sizes_vs_float64_forward(layers, dual, B, side):
     """Both precisions against arithmetic that is not this library's, at the sizes of BASELINE config 3 (SD3.5-medium widths, batch 2,
     64x64 latent = 1024 image tokens, 154 text tokens of width 4096): a model of four blocks (two with the extra self-attention, the
     last one discarding its context) and the full model of 24 blocks (13 dual) against the float64 forward written from the op list,
     which tests/test_oracle.py pins to the CPU oracle and to the compiled reference's outputs; and three blocks on one sample of the
-    headline shape (128x128 latent = 4096 image tokens). (The CPU oracle itself would need an hour for the second of these. The full
-    model at 1024x1024 is held to the fp32 path below, which this test and the golden vectors hold to the reference.)"""
+    headline shape (128x128 latent = 4096 image tokens). (The CPU oracle itself would need an hour for the second of these.) The full
+    24-block model on one sample of the headline shape takes the float64 forward some minutes on the host and runs only on request
+    (SD3_LONG_TESTS=1, pytest -s; two minutes on 16 host cores; measured: fp32 path 2.2e-6 rel-L2 and 9.4e-6 max-abs, bf16 path 4.3e-3)."""
     import dataclasses
     from sd3_c_amd.params import synthetic_params_numpy
     from test_oracle import dit64
@@ -71,11 +76,14 @@ def test_dit_at_512px_and_1024px_sizes_vs_float64_forward(layers, dual, B, side)
     k = dict(cfg=cfg, params=P, latent=rng.standard_normal((B, cfg.in_channels, side, side), dtype=np.float32),
              captions=rng.standard_normal((B, 154, cfg.captions_dim), dtype=np.float32), pooled=rng.standard_normal((B, cfg.pooled_dim), dtype=np.float32),
              timesteps=(rng.random(B) * 1000).astype(np.float32))
-    want = dit64(k["pooled"], k["captions"], k["latent"], k["timesteps"], P, cfg)
+    tick = (lambda l: print(f"float64 forward: block {l} done", flush=True)) if side * layers > 2000 else None
+    want = dit64(k["pooled"], k["captions"], k["latent"], k["timesteps"], P, cfg, tick)
     dP = dev_params(P)
-    out32 = run_gpu_dit(k, "fp32", dP)
+    out32, out16 = run_gpu_dit(k, "fp32", dP), run_gpu_dit(k, "bf16", dP)
+    print(f"{layers} blocks, batch {B}, {side}x{side} latent vs float64: fp32 path rel-L2 {rel_l2(out32, want):.3g} max-abs {max_abs(out32, want):.3g}, "
+          f"bf16 path rel-L2 {rel_l2(out16, want):.3g}", flush=True)
     assert rel_l2(out32, want) <= 2e-5 and max_abs(out32, want) <= F32_TOL   # measured 2e-6 and 3e-5 on 24 blocks
-    assert rel_l2(run_gpu_dit(k, "bf16", dP), want) <= BF16_REL_L2                # measured 4.2e-3 on 24 blocks
+    assert rel_l2(out16, want) <= BF16_REL_L2                                # measured 4.2e-3 on 24 blocks
 
 
 @pytest.mark.parametrize("file_dtype,shards", [("float32", 1), ("bfloat16", 3)])

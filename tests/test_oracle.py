@@ -206,7 +206,7 @@ def block64(y, c, x, P, NH, dual, qk, disc):
 
 
 # ---------------------------------------------------------------- float64 forward written from the op list (modules.cpp:1660-1752)
-def dit64(pooled, captions, latent, timesteps, P, cfg):
+def dit64(pooled, captions, latent, timesteps, P, cfg, progress=None):
     f = lambda n: P[n].astype(np.float64)  # noqa: E731
     silu = lambda a: a / (1 + np.exp(-a))  # noqa: E731
     pooled, captions, latent, t = (a.astype(np.float64) for a in (pooled, captions, latent, timesteps))
@@ -237,6 +237,8 @@ def dit64(pooled, captions, latent, timesteps, P, cfg):
         pre = f"transformer.{l}."
         Pl = {n[len(pre):]: v for n, v in P.items() if n.startswith(pre)}
         c, x = block64(y, c, x, Pl, cfg.attn_heads, l in cfg.dual_attention_layers, cfg.use_qk_norm, l == cfg.num_layers - 1)
+        if progress:
+            progress(l)
     m = x.mean(-1, keepdims=True)
     xh = (x - m) / np.sqrt(((x - m) ** 2).mean(-1, keepdims=True) + 1e-5)
     scale, shift = np.split(y @ f("ada_ln_out.linear.weight") + f("ada_ln_out.linear.bias"), 2, -1)   # chunk 0 = scale, chunk 1 = shift
