@@ -172,6 +172,20 @@ def test_dit_batch_sweep_at_the_benchmark_shape(B):
         assert rel_l2(run_gpu_dit(k1, "bf16", P)[0], o16[-1]) <= 1e-5
 
 
+@pytest.mark.parametrize("B,h,w,Tc", [(1, 256, 256, 154), (1, 192, 80, 77), (3, 34, 62, 333)])
+def test_dit_other_image_sizes_bf16_vs_fp32_sd35_medium(B, h, w, Tc):
+    """The full model away from the benchmark's sizes: a 2048x2048 image (256x256 latent, 16384 image tokens: four times the headline
+    sequence, 257 key tiles per attention item), a non-square 1536x640 one with 77 text tokens, and a batch of three with a grid and a
+    text length that are multiples of no tile (17 x 31 patches, 333 text tokens)."""
+    cfg = sd35_medium()
+    P = _synthetic_device_params(cfg, 5)
+    k = _inputs(cfg, B, Tc, h, w, 40 + B)
+    o32 = run_gpu_dit(k, "fp32", P)
+    o16 = run_gpu_dit(k, "bf16", P)
+    assert np.isfinite(o32).all() and np.isfinite(o16).all()
+    assert rel_l2(o16, o32) <= BF16_REL_L2   # measured 4.4e-3, 5.0e-3, 4.9e-3
+
+
 def test_dit_batch_beyond_the_limit_is_rejected():
     from sd3_c_amd import lib as L_
     cfg = DiTConfig(num_layers=1, dual_attention_layers=(), emb_dim=128, attn_heads=2, pooled_dim=64, captions_dim=64, pos_embed_max_size=16, base_height=8)
