@@ -602,7 +602,6 @@ int check_block_dims(const Dims& d, int prec) {
     if (d.B <= 0 || d.Tc < 0 || d.Tx <= 0 || d.C <= 0 || d.NH <= 0 || d.E <= 0)
         return fail(SD3_ERR_INVALID_ARG, "block: sizes must be positive (B=%d Tc=%d Tx=%d emb_dim=%d heads=%d mlp_expand=%d)", d.B, d.Tc, d.Tx, d.C, d.NH, d.E);
     if (d.C % d.NH) return fail(SD3_ERR_INVALID_ARG, "block: emb_dim %d is not divisible by attn_heads %d", d.C, d.NH);
-    if (d.B > 8) return fail(SD3_ERR_UNSUPPORTED, "block: batch %d > 8", d.B);
     if (prec < SD3_PREC_F32 || prec > SD3_PREC_BF16_FP8_TENSOR) return fail(SD3_ERR_INVALID_ARG, "unknown precision %d", prec);
     if (is_bf(prec) && (d.HS != 64 || d.C % 64)) return fail(SD3_ERR_UNSUPPORTED, "bf16 path needs head_dim 64 and emb_dim %% 64 == 0");
     if (fp8_kind(prec) && (d.C % 128)) return fail(SD3_ERR_UNSUPPORTED, "fp8 MLPs need emb_dim %% 128 == 0");

@@ -1,7 +1,9 @@
-// Linear layers whose left operand has at most 8 rows (the batch): the adaLN modulation projections
+// Linear layers whose left operand has few rows (the batch; eight per launch): the adaLN modulation projections
 // (modules.cpp:1384-1501 compute them one 1536-column chunk at a time with partial_linear), the timestep and
 // pooled-text MLPs (modules.cpp:1664-1671). They are pure weight streaming, so one launch covers a whole list
 // of weight matrices ("jobs") and reads every weight element exactly once, N-contiguous as the reference stores it.
+#include <vector>
+
 #include "common.hpp"
 
 namespace sd3 {
@@ -114,7 +116,16 @@ static void launch_small(const float* x, int m_real, int K, const SmallLinearJob
 
 int small_linear_batched(const float* x, int M, int K, const SmallLinearJob* jobs_host, int n_jobs, int w_is_bf16, int act, hipStream_t st) {
     if (M <= 0 || n_jobs <= 0) return SD3_OK;
-    if (M > 8) return fail(SD3_ERR_UNSUPPORTED, "small_linear: at most 8 rows (got %d)", M);
+    if (M > 8) {
+        // more than eight rows (the reference's own block test runs a batch of 16, module_tests/dit_block.py:12): eight at a time, the
+        // weights streamed once per group of rows
+        std::vector<SmallLinearJob> part(jobs_host, jobs_host + n_jobs);
+        for (int m0 = 0; m0 < M; m0 += 8) {
+            for (int i = 0; i < n_jobs; i++) part[i].out = jobs_host[i].out ? jobs_host[i].out + (long long)m0 * jobs_host[i].N : nullptr;
+            SD3_TRY(small_linear_batched(x + (long long)m0 * K, M - m0 < 8 ? M - m0 : 8, K, part.data(), n_jobs, w_is_bf16, act, st));
+        }
+        return SD3_OK;
+    }
     if ((size_t)(K > 1024 ? K : 1024) * 8 * sizeof(float) > 65536 && M > 4)
         return fail(SD3_ERR_UNSUPPORTED, "small_linear: K=%d too large for %d rows", K, M);
     if (K > 4096) return fail(SD3_ERR_UNSUPPORTED, "small_linear: K=%d too large", K);

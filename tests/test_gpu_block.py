@@ -172,6 +172,28 @@ def test_block_bf16_at_512px_and_1024px_token_counts_vs_float64(dual, discard, B
         assert np.array_equal(c16, k["c"])
 
 
+def test_block_at_the_sizes_of_the_reference_block_test():
+    """module_tests/dit_block.py:9-22: batch 16, 512 image + 154 text tokens, width 768, 12 heads of 64, mlp_expand 2, the extra
+    self-attention and qk-norm on, y = silu(randn). The reference script only prints its differences; here both precisions are held
+    to the float64 statement of the block (the CPU oracle would need minutes), and the sixteen batch elements go through the
+    modulation projections in two groups of eight."""
+    rng = np.random.Generator(np.random.Philox(81))
+    B, Tc, Tx, C, NH, E = 16, 154, 512, 768, 12, 2
+    params = synthetic_params_numpy(block_param_shapes(C, E, True, True, False, C // NH), 82, 0.03, 0.03)
+    y = rng.standard_normal((B, C), dtype=np.float32)
+    k = dict(y=(y / (1 + np.exp(-y))).astype(np.float32), c=rng.standard_normal((B, Tc, C), dtype=np.float32),
+             x=rng.standard_normal((B, Tx, C), dtype=np.float32), params=params, NH=NH, mlp_expand=E, use_dual=True, use_qk_norm=True,
+             discard_context=False)
+    c64, x64 = block64(k["y"], k["c"], k["x"], k["params"], NH, True, True, False)
+    c32, x32 = run_gpu_block(k, "fp32")
+    assert max_abs(x32, x64) <= F32_TOL and max_abs(c32, c64) <= F32_TOL
+    c16, x16 = run_gpu_block(k, "bf16")
+    assert rel_l2(x16, x64) <= BF16_REL_L2 and rel_l2(c16, c64) <= BF16_REL_L2
+    # every element separately (a wrong row of modulation vectors for elements 8..15 would hide in a norm over the batch)
+    for b in range(B):
+        assert rel_l2(x16[b], x64[b]) <= BF16_REL_L2 and max_abs(x32[b], x64[b]) <= F32_TOL, b
+
+
 def test_block_zero_gates_is_identity_on_gpu():
     k = _wide_case(1, 77, 256, True, False, 31)
     P = dict(k["params"])

@@ -186,12 +186,21 @@ def test_dit_other_image_sizes_bf16_vs_fp32_sd35_medium(B, h, w, Tc):
     assert rel_l2(o16, o32) <= BF16_REL_L2   # measured 4.4e-3, 5.0e-3, 4.9e-3
 
 
-def test_dit_batch_beyond_the_limit_is_rejected():
-    from sd3_c_amd import lib as L_
-    cfg = DiTConfig(num_layers=1, dual_attention_layers=(), emb_dim=128, attn_heads=2, pooled_dim=64, captions_dim=64, pos_embed_max_size=16, base_height=8)
+@pytest.mark.parametrize("B", [9, 16])
+def test_dit_batches_beyond_eight(B):
+    """More batch elements than one launch of the modulation projections takes (eight): the forward against the CPU oracle, and every
+    element equal to the same element computed alone."""
+    cfg = DiTConfig(num_layers=2, dual_attention_layers=(0,), emb_dim=128, attn_heads=2, pooled_dim=64, captions_dim=64, pos_embed_max_size=16, base_height=8)
     P = _synthetic_device_params(cfg, 3)
-    with pytest.raises(L_.Sd3Error, match="batch"):
-        run_gpu_dit(_inputs(cfg, 9, 2, 8, 8, 4), "bf16", P)
+    k = _inputs(cfg, B, 3, 8, 12, 4)
+    o32 = run_gpu_dit(k, "fp32", P)
+    host_P = {n: host(v) for n, v in P.items()}
+    assert max_abs(o32, ol.orc_dit_forward(k["pooled"], k["captions"], k["latent"], k["timesteps"], host_P, cfg)) <= F32_TOL
+    o16 = run_gpu_dit(k, "bf16", P)
+    assert rel_l2(o16, o32) <= BF16_REL_L2
+    for b in (0, 7, 8, B - 1):
+        k1 = dict(k, latent=k["latent"][b:b + 1], captions=k["captions"][b:b + 1], pooled=k["pooled"][b:b + 1], timesteps=k["timesteps"][b:b + 1])
+        assert rel_l2(run_gpu_dit(k1, "bf16", P)[0], o16[b]) <= 1e-5, b
 
 
 def test_dit_ragged_shapes_bf16_vs_fp32():
