@@ -172,15 +172,24 @@ def mha(query, key, value, num_heads):
     return out
 
 
-def mlp(input, W1, b1, W2, b2, activation):
-    """modules.cpp:1167 MLP with the activation given by name ("silu" or "gelu_tanh")."""
+def mlp(input, W1, b1, W2, b2, activation, B=None, C_in=None, C_hid=None, C_out=None):
+    """modules.cpp:1167 MLP: act(x @ W1 + b1) @ W2 + b2, argument list of the reference's binding (the four sizes may be left out: they
+    follow from the weights). `activation` by the reference's names, "GELU" / "gelu" (the tanh form) or "silu" / "SILU" / "SiLU", or
+    "gelu_tanh". (The reference's binding sets the activation to SiLU whatever the name, modules.cpp:1190-1192; here the name is
+    honoured, as in the raw-pointer mlp of modules.cpp:1120 that the forward path uses.)"""
     x = _dev(input, "input")
     Cin, Chid = W1.shape
     Cout = W2.shape[1]
     rows = x.numel() // Cin
+    for given, actual, what in ((B, rows, "B"), (C_in, Cin, "C_in"), (C_hid, Chid, "C_hid"), (C_out, Cout, "C_out")):
+        if given is not None and int(given) != actual:
+            raise ValueError(f"mlp: {what}={given} does not match the tensors ({actual})")
     h = torch.empty((rows, Chid), device=x.device)
     out = torch.empty(x.shape[:-1] + (Cout,), device=x.device)
-    act = {"silu": L.ACT_SILU, "gelu_tanh": L.ACT_GELU_TANH}[activation]
+    names = {"silu": L.ACT_SILU, "SILU": L.ACT_SILU, "SiLU": L.ACT_SILU, "gelu_tanh": L.ACT_GELU_TANH, "GELU": L.ACT_GELU_TANH, "gelu": L.ACT_GELU_TANH}
+    if activation not in names:
+        raise ValueError(f"mlp: unknown activation {activation!r}")
+    act = names[activation]
     L.call("sd3_mlp", _p(x), _p(out), _p(h), _p(_dev(W1, "W1")), _p(_dev(b1, "b1")), _p(_dev(W2, "W2")), _p(_dev(b2, "b2")), rows, Cin, Chid, Cout, act,
            _stream())
     return out
