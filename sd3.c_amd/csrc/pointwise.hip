@@ -147,7 +147,7 @@ __global__ void __launch_bounds__(256) ln_mod_generic_kernel(const float* __rest
 template <typename OutT>
 static bool ln_seg_vectorisable(const LnSegDev<OutT>& g, int C) {
     auto al = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
-    return (C % 4 == 0) && (C <= 2048) && (g.mod_ld % 4 == 0) && al(g.x) && al(g.out) && al(g.out2) && al(g.shift) && al(g.scale) && al(g.shift2) &&
+    return (C % 4 == 0) && (C <= 3072) && (g.mod_ld % 4 == 0) && al(g.x) && al(g.out) && al(g.out2) && al(g.shift) && al(g.scale) && al(g.shift2) &&
            al(g.scale2);
 }
 template <typename OutT>
@@ -160,7 +160,8 @@ static int ln_mod_launch_vec(const LnSegPair<OutT>& segs, float eps, int C, hipS
     case N:                                                                                  \
         hipLaunchKernelGGL((ln_mod_vec_kernel<OutT, N>), grid, block, 0, st, segs, eps, C); \
         break;
-    switch (nv) { SD3_LN_CASE(1) SD3_LN_CASE(2) SD3_LN_CASE(3) SD3_LN_CASE(4) SD3_LN_CASE(5) SD3_LN_CASE(6) SD3_LN_CASE(7) SD3_LN_CASE(8) }
+    switch (nv) { SD3_LN_CASE(1) SD3_LN_CASE(2) SD3_LN_CASE(3) SD3_LN_CASE(4) SD3_LN_CASE(5) SD3_LN_CASE(6) SD3_LN_CASE(7) SD3_LN_CASE(8)
+                  SD3_LN_CASE(9) SD3_LN_CASE(10) SD3_LN_CASE(11) SD3_LN_CASE(12) }
 #undef SD3_LN_CASE
     return launch_status("layernorm_modulate");
 }

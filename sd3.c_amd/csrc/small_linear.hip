@@ -116,19 +116,19 @@ static void launch_small(const float* x, int m_real, int K, const SmallLinearJob
 
 int small_linear_batched(const float* x, int M, int K, const SmallLinearJob* jobs_host, int n_jobs, int w_is_bf16, int act, hipStream_t st) {
     if (M <= 0 || n_jobs <= 0) return SD3_OK;
-    if (M > 8) {
-        // more than eight rows (the reference's own block test runs a batch of 16, module_tests/dit_block.py:12): eight at a time, the
-        // weights streamed once per group of rows
+    if (K > 4096) return fail(SD3_ERR_UNSUPPORTED, "small_linear: K=%d too large", K);
+    // rows per launch: eight, or four when eight transposed rows of x do not fit the 64 KB of LDS a workgroup may use (K > 2048)
+    const int group = ((size_t)(K > 1024 ? K : 1024) * 8 * sizeof(float) > 65536) ? 4 : 8;
+    if (M > group) {
+        // more rows than that (the reference's own block test runs a batch of 16, module_tests/dit_block.py:12): a group at a time, the
+        // weights streamed once per group
         std::vector<SmallLinearJob> part(jobs_host, jobs_host + n_jobs);
-        for (int m0 = 0; m0 < M; m0 += 8) {
+        for (int m0 = 0; m0 < M; m0 += group) {
             for (int i = 0; i < n_jobs; i++) part[i].out = jobs_host[i].out ? jobs_host[i].out + (long long)m0 * jobs_host[i].N : nullptr;
-            SD3_TRY(small_linear_batched(x + (long long)m0 * K, M - m0 < 8 ? M - m0 : 8, K, part.data(), n_jobs, w_is_bf16, act, st));
+            SD3_TRY(small_linear_batched(x + (long long)m0 * K, M - m0 < group ? M - m0 : group, K, part.data(), n_jobs, w_is_bf16, act, st));
         }
         return SD3_OK;
     }
-    if ((size_t)(K > 1024 ? K : 1024) * 8 * sizeof(float) > 65536 && M > 4)
-        return fail(SD3_ERR_UNSUPPORTED, "small_linear: K=%d too large for %d rows", K, M);
-    if (K > 4096) return fail(SD3_ERR_UNSUPPORTED, "small_linear: K=%d too large", K);
     const int esz = w_is_bf16 ? 2 : 4;
     for (int base = 0; base < n_jobs; base += 16) {
         const int n = (n_jobs - base) < 16 ? (n_jobs - base) : 16;

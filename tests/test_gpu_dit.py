@@ -311,3 +311,22 @@ def test_warm_forward_is_graph_capturable_and_replays_bit_identically():
             graph.replay()
             torch.cuda.synchronize()
             assert torch.equal(out, want) and torch.equal(step_out, want_step), (precision, i)
+
+
+@pytest.mark.parametrize("B", [2, 6])
+def test_dit_at_the_width_of_sd35_large(B):
+    """The forward is generic in its sizes (modules.cpp:1605-1613): a model of the SD3.5-large widths (38 heads of 64 = width 2432,
+    three blocks, the first with the extra self-attention) on a 32x32 latent with 20 text tokens: fp32 path against the float64 forward,
+    bf16 path against the same. (Width 2432 takes the modulation projections in groups of four batch elements and the LayerNorm rows
+    through ten 16-byte loads per lane.)"""
+    from sd3_c_amd.params import synthetic_params_numpy
+    from test_oracle import dit64
+    cfg = DiTConfig(num_layers=3, dual_attention_layers=(0,), emb_dim=2432, attn_heads=38, pooled_dim=2048, captions_dim=4096, pos_embed_max_size=192,
+                    base_height=64)
+    P = synthetic_params_numpy(dit_param_shapes(cfg), 61, 0.02, 0.02)
+    k = _inputs(cfg, B, 20, 32, 32, 62)
+    want = dit64(k["pooled"], k["captions"], k["latent"], k["timesteps"], P, cfg)
+    dP = dev_params(P)
+    o32 = run_gpu_dit(k, "fp32", dP)
+    assert rel_l2(o32, want) <= 2e-5 and max_abs(o32, want) <= F32_TOL
+    assert rel_l2(run_gpu_dit(k, "bf16", dP), want) <= BF16_REL_L2
