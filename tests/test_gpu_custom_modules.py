@@ -50,6 +50,27 @@ def test_block_called_like_module_tests_dit_block_py(name):
     assert x2 is xd and torch.equal(xd.cpu(), x)
 
 
+def test_block_at_the_sizes_of_module_tests_dit_block_py():
+    """module_tests/dit_block.py:9-66 with its own sizes (batch 16, 512 image + 154 text tokens, width 768, 12 heads, mlp_expand 2, extra
+    self-attention and qk-norm on, y = silu(randn)), its two calls -- host tensors through Dit_block, device tensors through
+    DiT_block_cuda -- and its checks (max difference of c_out and x_out), here against the float64 statement of the block."""
+    from sd3_c_amd.params import block_param_shapes, synthetic_params_numpy
+    from test_oracle import block64
+    B, Tc, Tx, emb_dim, attn_heads, mlp_expand = 16, 77 + 77, 512, 768, 12, 2
+    torch.manual_seed(5)
+    P = synthetic_params_numpy(block_param_shapes(emb_dim, mlp_expand, True, True, False, emb_dim // attn_heads), 6, emb_dim ** -0.5 / 3 ** 0.5, 0.02)
+    params = {n: torch.from_numpy(v) for n, v in P.items()}
+    x, y, c = torch.randn((B, Tx, emb_dim)), torch.nn.functional.silu(torch.randn((B, emb_dim))), torch.randn((B, Tc, emb_dim))
+    c_true, x_true = block64(y.numpy(), c.numpy(), x.numpy(), P, attn_heads, True, True, False)
+    c_clone, x_clone, y_clone = c.clone().to("cuda"), x.clone().to("cuda"), y.clone().to("cuda")
+    c_out, x_out = F.Dit_block(y, c, x, params, B, Tc, Tx, emb_dim, attn_heads, mlp_expand, True, True, False)
+    assert max_abs(c_out.numpy(), c_true) <= F32_TOL and max_abs(x_out.numpy(), x_true) <= F32_TOL
+    params_cuda = {n: v.to("cuda") for n, v in params.items()}
+    c_out_cuda, x_out_cuda = F.DiT_block_cuda(y_clone, c_clone, x_clone, params_cuda, B, Tc, Tx, emb_dim, attn_heads, mlp_expand, True, True, False)
+    assert max_abs(c_out_cuda.cpu().numpy(), c_true) <= F32_TOL and max_abs(x_out_cuda.cpu().numpy(), x_true) <= F32_TOL
+    F.release()
+
+
 def test_module_level_precision_switch_reaches_the_bf16_path():
     """A script written against the reference's signatures selects the bf16 path with F.PRECISION; results then differ from the
     fp32 ones in the low bits only (and the switch goes back)."""
