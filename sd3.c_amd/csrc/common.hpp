@@ -192,6 +192,7 @@ struct SmallLinearJob {
     int ldw;  // row stride of W
     int n0;   // first column
 };
+constexpr int SMALL_LINEAR_JOBS_PER_LAUNCH = 64;
 int small_linear_batched(const float* x, int M, int K, const SmallLinearJob* jobs_host, int n_jobs, int w_is_bf16, int act /* -1 none */,
                          hipStream_t st);
 

@@ -350,7 +350,7 @@ int ada_jobs_run(sd3_ctx* ctx, int prec, const float* y, int B, int C, std::vect
     }
     double bytes = 0;
     for (auto& j : jobs) bytes += (double)C * j.N * (is_bf(prec) ? 2 : 4) + (double)B * j.N * 4;
-    ProfScope ps(ctx, SD3_PROF_ADALN, bytes, ((long long)jobs.size() + 15) / 16);  // one kernel per 16 weight matrices
+    ProfScope ps(ctx, SD3_PROF_ADALN, bytes, ((long long)jobs.size() + SMALL_LINEAR_JOBS_PER_LAUNCH - 1) / SMALL_LINEAR_JOBS_PER_LAUNCH);
     return small_linear_batched(y, B, C, jobs.data(), (int)jobs.size(), is_bf(prec), -1, ctx->stream);
 }
 

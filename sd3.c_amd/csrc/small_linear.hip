@@ -32,7 +32,7 @@ struct WLoad<bf16_t> {
 // x is staged transposed in LDS (xs[k][m]) so that a thread reads its M inputs for one k with wide LDS loads.
 // Jobs travel as a kernel argument (no device-side table to keep coherent with the host).
 struct SmallLinearJobPack {
-    SmallLinearJob j[16];
+    SmallLinearJob j[SMALL_LINEAR_JOBS_PER_LAUNCH];  // 64 x 40 bytes of kernel arguments: the 49 projections of a 24-block forward in one launch
 };
 
 template <int M, typename WT, bool VEC>
@@ -130,8 +130,9 @@ int small_linear_batched(const float* x, int M, int K, const SmallLinearJob* job
         return SD3_OK;
     }
     const int esz = w_is_bf16 ? 2 : 4;
-    for (int base = 0; base < n_jobs; base += 16) {
-        const int n = (n_jobs - base) < 16 ? (n_jobs - base) : 16;
+    constexpr int PER = SMALL_LINEAR_JOBS_PER_LAUNCH;
+    for (int base = 0; base < n_jobs; base += PER) {
+        const int n = (n_jobs - base) < PER ? (n_jobs - base) : PER;
         SmallLinearJobPack pack;
         int max_N = 0;
         bool vec = true;
@@ -141,7 +142,7 @@ int small_linear_batched(const float* x, int M, int K, const SmallLinearJob* job
             if (j.N > max_N) max_N = j.N;
             if ((j.N % 4) || (j.ldw % 4) || (j.n0 % 4) || ((reinterpret_cast<uintptr_t>(j.W) % (4 * esz)) != 0)) vec = false;
         }
-        for (int i = n; i < 16; i++) pack.j[i] = SmallLinearJob{nullptr, nullptr, nullptr, 0, 0, 0};
+        for (int i = n; i < PER; i++) pack.j[i] = SmallLinearJob{nullptr, nullptr, nullptr, 0, 0, 0};
         if (max_N == 0) continue;
         if (M == 1) launch_small<1>(x, M, K, pack, n, max_N, w_is_bf16, vec, act, st);
         else if (M == 2) launch_small<2>(x, M, K, pack, n, max_N, w_is_bf16, vec, act, st);
