@@ -191,8 +191,10 @@ struct SmallLinearJob {
     int N;    // columns of this job
     int ldw;  // row stride of W
     int n0;   // first column
+    const float* x = nullptr;  // this job's own left operand (M, K) instead of the launch's, or null
+    int K = 0;                 // its depth (with x)
 };
-constexpr int SMALL_LINEAR_JOBS_PER_LAUNCH = 64;
+constexpr int SMALL_LINEAR_JOBS_PER_LAUNCH = 52;
 int small_linear_batched(const float* x, int M, int K, const SmallLinearJob* jobs_host, int n_jobs, int w_is_bf16, int act /* -1 none */,
                          hipStream_t st);
 

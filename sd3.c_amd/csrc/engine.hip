@@ -1107,10 +1107,11 @@ static int dit_forward_impl(sd3_ctx* ctx, const float* pooled, const float* capt
     }
 
     // ---- workspace
-    auto layout = [&](Bump& b, float** temb, float** h1, float** yt, float** yp, float** y, float** c, float** x, void** cap_in, void** patches,
+    auto layout = [&](Bump& b, float** temb, float** h1, float** h2, float** yt, float** yp, float** y, float** c, float** x, void** cap_in, void** patches,
                       float** ada_all, float** ada_out, float** tokens) {
         *temb = b.take<float>((size_t)B * 256);
         *h1 = b.take<float>((size_t)B * C);
+        *h2 = b.take<float>((size_t)B * C);
         *yt = b.take<float>((size_t)B * C);
         *yp = b.take<float>((size_t)B * C);
         *y = b.take<float>((size_t)B * C);
@@ -1122,26 +1123,23 @@ static int dit_forward_impl(sd3_ctx* ctx, const float* pooled, const float* capt
         *ada_out = b.take<float>((size_t)B * 2 * C);
         *tokens = b.take<float>((size_t)B * Tx * PPC);
     };
-    float *temb, *h1, *yt, *yp, *y, *c, *x, *ada_all, *ada_out, *tokens;
+    float *temb, *h1, *h2, *yt, *yp, *y, *c, *x, *ada_all, *ada_out, *tokens;
     void *cap_in, *patches;
     Bump probe(nullptr, 0);
-    layout(probe, &temb, &h1, &yt, &yp, &y, &c, &x, &cap_in, &patches, &ada_all, &ada_out, &tokens);
+    layout(probe, &temb, &h1, &h2, &yt, &yp, &y, &c, &x, &cap_in, &patches, &ada_all, &ada_out, &tokens);
     SD3_TRY(ensure_workspace(ctx, probe.off + block_workspace_bytes(dmax, precision)));
     Bump ws(ctx->ws, ctx->ws_bytes);
-    layout(ws, &temb, &h1, &yt, &yp, &y, &c, &x, &cap_in, &patches, &ada_all, &ada_out, &tokens);
+    layout(ws, &temb, &h1, &h2, &yt, &yp, &y, &c, &x, &cap_in, &patches, &ada_all, &ada_out, &tokens);
     const size_t block_ws_off = ws.off;
 
     // ---- y = silu(MLP(t_emb) + MLP(pooled)) (modules.cpp:1663-1675); weights stay fp32 here: 8 MB read once
     SD3_TRY(timestep_embedding(timesteps, temb, B, 256, st));
     {
-        SmallLinearJob j1{t_w0, t_b0, h1, C, C, 0};
-        SD3_TRY(small_linear_batched(temb, B, 256, &j1, 1, 0, SD3_ACT_SILU, st));
-        SmallLinearJob j2{t_w2, t_b2, yt, C, C, 0};
-        SD3_TRY(small_linear_batched(h1, B, C, &j2, 1, 0, -1, st));
-        SmallLinearJob j3{p_w0, p_b0, h1, C, C, 0};
-        SD3_TRY(small_linear_batched(pooled, B, pooled_dim, &j3, 1, 0, SD3_ACT_SILU, st));
-        SmallLinearJob j4{p_w2, p_b2, yp, C, C, 0};
-        SD3_TRY(small_linear_batched(h1, B, C, &j4, 1, 0, -1, st));
+        // the two MLPs side by side: both first layers in one launch (each job brings its own input), then both second layers
+        const SmallLinearJob first[2] = {{t_w0, t_b0, h1, C, C, 0, temb, 256}, {p_w0, p_b0, h2, C, C, 0, pooled, pooled_dim}};
+        SD3_TRY(small_linear_batched(nullptr, B, 0, first, 2, 0, SD3_ACT_SILU, st));
+        const SmallLinearJob second[2] = {{t_w2, t_b2, yt, C, C, 0, h1, C}, {p_w2, p_b2, yp, C, C, 0, h2, C}};
+        SD3_TRY(small_linear_batched(nullptr, B, 0, second, 2, 0, -1, st));
         SD3_TRY(add_silu_op(yt, yp, y, (long long)B * C, st));
     }
     // ---- c = captions @ W + b (modules.cpp:1678)

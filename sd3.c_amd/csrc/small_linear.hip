@@ -32,15 +32,17 @@ struct WLoad<bf16_t> {
 // x is staged transposed in LDS (xs[k][m]) so that a thread reads its M inputs for one k with wide LDS loads.
 // Jobs travel as a kernel argument (no device-side table to keep coherent with the host).
 struct SmallLinearJobPack {
-    SmallLinearJob j[SMALL_LINEAR_JOBS_PER_LAUNCH];  // 64 x 40 bytes of kernel arguments: the 49 projections of a 24-block forward in one launch
+    SmallLinearJob j[SMALL_LINEAR_JOBS_PER_LAUNCH];  // 52 x 56 bytes of kernel arguments: the 49 projections of a 24-block forward in one launch
 };
 
 template <int M, typename WT, bool VEC>
-__global__ void __launch_bounds__(256) small_linear_kernel(const float* __restrict__ x, int m_real, int K, const SmallLinearJobPack jobs, int act) {
+__global__ void __launch_bounds__(256) small_linear_kernel(const float* __restrict__ x_all, int m_real, int K_all, const SmallLinearJobPack jobs, int act) {
     extern __shared__ float smem[];
     const SmallLinearJob job = jobs.j[blockIdx.y];
     const int col_base = blockIdx.x * 128;
     if (col_base >= job.N) return;
+    const float* __restrict__ x = job.x ? job.x : x_all;  // (uniform over the workgroup)
+    const int K = job.x ? job.K : K_all;
     const int tid = threadIdx.x;
 #pragma unroll
     for (int m = 0; m < M; m++)
@@ -100,10 +102,10 @@ __global__ void __launch_bounds__(256) small_linear_kernel(const float* __restri
 }
 
 template <int M>
-static void launch_small(const float* x, int m_real, int K, const SmallLinearJobPack& jobs, int n_jobs, int max_N, int w_is_bf16, bool vec, int act,
+static void launch_small(const float* x, int m_real, int K, int K_max, const SmallLinearJobPack& jobs, int n_jobs, int max_N, int w_is_bf16, bool vec, int act,
                          hipStream_t st) {
     dim3 grid((max_N + 127) / 128, n_jobs), block(256);
-    const int kk = K > 1024 ? K : 1024;
+    const int kk = K_max > 1024 ? K_max : 1024;
     const size_t smem = (size_t)kk * M * sizeof(float);
     if (w_is_bf16) {
         if (vec) hipLaunchKernelGGL((small_linear_kernel<M, bf16_t, true>), grid, block, smem, st, x, m_real, K, jobs, act);
@@ -116,7 +118,12 @@ static void launch_small(const float* x, int m_real, int K, const SmallLinearJob
 
 int small_linear_batched(const float* x, int M, int K, const SmallLinearJob* jobs_host, int n_jobs, int w_is_bf16, int act, hipStream_t st) {
     if (M <= 0 || n_jobs <= 0) return SD3_OK;
-    if (K > 4096) return fail(SD3_ERR_UNSUPPORTED, "small_linear: K=%d too large", K);
+    const int K_launch = K;  // depth of the launch's own x (jobs may bring theirs)
+    for (int i = 0; i < n_jobs; i++) {
+        if (!jobs_host[i].x && !x) return fail(SD3_ERR_INVALID_ARG, "small_linear: job %d has no left operand", i);
+        if (jobs_host[i].x && jobs_host[i].K > K) K = jobs_host[i].K;  // from here on K is the largest depth of the launch (LDS size)
+    }
+    if (K <= 0 || K > 4096) return fail(SD3_ERR_UNSUPPORTED, "small_linear: K=%d out of range", K);
     // rows per launch: eight, or four when eight transposed rows of x do not fit the 64 KB of LDS a workgroup may use (K > 2048)
     const int group = ((size_t)(K > 1024 ? K : 1024) * 8 * sizeof(float) > 65536) ? 4 : 8;
     if (M > group) {
@@ -124,8 +131,11 @@ int small_linear_batched(const float* x, int M, int K, const SmallLinearJob* job
         // weights streamed once per group
         std::vector<SmallLinearJob> part(jobs_host, jobs_host + n_jobs);
         for (int m0 = 0; m0 < M; m0 += group) {
-            for (int i = 0; i < n_jobs; i++) part[i].out = jobs_host[i].out ? jobs_host[i].out + (long long)m0 * jobs_host[i].N : nullptr;
-            SD3_TRY(small_linear_batched(x + (long long)m0 * K, M - m0 < group ? M - m0 : group, K, part.data(), n_jobs, w_is_bf16, act, st));
+            for (int i = 0; i < n_jobs; i++) {
+                part[i].out = jobs_host[i].out ? jobs_host[i].out + (long long)m0 * jobs_host[i].N : nullptr;
+                part[i].x = jobs_host[i].x ? jobs_host[i].x + (long long)m0 * jobs_host[i].K : nullptr;
+            }
+            SD3_TRY(small_linear_batched(x ? x + (long long)m0 * K_launch : nullptr, M - m0 < group ? M - m0 : group, K_launch, part.data(), n_jobs, w_is_bf16, act, st));
         }
         return SD3_OK;
     }
@@ -142,12 +152,12 @@ int small_linear_batched(const float* x, int M, int K, const SmallLinearJob* job
             if (j.N > max_N) max_N = j.N;
             if ((j.N % 4) || (j.ldw % 4) || (j.n0 % 4) || ((reinterpret_cast<uintptr_t>(j.W) % (4 * esz)) != 0)) vec = false;
         }
-        for (int i = n; i < PER; i++) pack.j[i] = SmallLinearJob{nullptr, nullptr, nullptr, 0, 0, 0};
+        for (int i = n; i < PER; i++) pack.j[i] = SmallLinearJob{nullptr, nullptr, nullptr, 0, 0, 0, nullptr, 0};
         if (max_N == 0) continue;
-        if (M == 1) launch_small<1>(x, M, K, pack, n, max_N, w_is_bf16, vec, act, st);
-        else if (M == 2) launch_small<2>(x, M, K, pack, n, max_N, w_is_bf16, vec, act, st);
-        else if (M <= 4) launch_small<4>(x, M, K, pack, n, max_N, w_is_bf16, vec, act, st);
-        else launch_small<8>(x, M, K, pack, n, max_N, w_is_bf16, vec, act, st);
+        if (M == 1) launch_small<1>(x, M, K_launch, K, pack, n, max_N, w_is_bf16, vec, act, st);
+        else if (M == 2) launch_small<2>(x, M, K_launch, K, pack, n, max_N, w_is_bf16, vec, act, st);
+        else if (M <= 4) launch_small<4>(x, M, K_launch, K, pack, n, max_N, w_is_bf16, vec, act, st);
+        else launch_small<8>(x, M, K_launch, K, pack, n, max_N, w_is_bf16, vec, act, st);
         SD3_TRY(launch_status("small_linear"));
     }
     return SD3_OK;
