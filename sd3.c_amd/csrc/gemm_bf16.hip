@@ -195,6 +195,7 @@ __device__ __forceinline__ void gemm_tile(const Prob& pr, const int wg, char* sm
     const int e_row = lane_on ? lane / CPR : 0, e_col = lane_on ? (lane % CPR) * 4 : 0;
     const int n0 = n_blk + wn * WNC + e_col;
     const bool vec_ok = ((N & 3) == 0) && ((ldc & 3) == 0);
+    const bool table_vec = EPI == EPI_BIAS_ROWADD && ((epi.gate_ld & 3) == 0) && ((reinterpret_cast<uintptr_t>(epi.table) & 15) == 0);
     const int nvalid = lane_on ? min(4, N - n0) : 0;  // <= 0 for lanes beyond the last column (and for lanes that sit out)
     // batch index of a row without a division per row: the tile starts in batch b0 and crosses a boundary every rpb rows
     const int rpb = epi.rows_per_batch, b0 = m_blk / rpb;
@@ -468,9 +469,14 @@ __device__ __forceinline__ void gemm_tile(const Prob& pr, const int wg, char* sm
                     }
                 } else if (EPI == EPI_BIAS_ROWADD) {
                     const float* t = epi.table + (long long)(m % rpb) * epi.gate_ld + n0;
+                    if (vec_ok && table_vec) {
+                        const float4 t4 = *reinterpret_cast<const float4*>(t);
+                        v[0] += t4.x; v[1] += t4.y; v[2] += t4.z; v[3] += t4.w;
+                    } else {
 #pragma unroll
-                    for (int c = 0; c < 4; c++)
-                        if (c < nvalid) v[c] += t[c];
+                        for (int c = 0; c < 4; c++)
+                            if (c < nvalid) v[c] += t[c];
+                    }
                 }
                 if constexpr (EPI == EPI_QKV_NORM && WNC % 64 == 0) {
                     // 16 consecutive lanes hold 64 consecutive columns of this row = one head of one token (modules.cpp:192-198, fused)
