@@ -221,6 +221,11 @@ __device__ __forceinline__ void gemm_tile(const Prob& pr, const int wg, char* sm
         // (it would be waited for at once); B fragments: two buffers
         // (one such row block for the large tiles: more of them cost registers, which the gated fp32 epilogue then spills)
         constexpr int TAIL = MI >= 6 ? 1 : MI / 2, HEAD = MI - TAIL;
+        // Where the direct loads of the next-but-one tile go among the 32 matrix instructions of a tile's last step: one behind every
+        // second instruction, from the seventh on (behind the fragment reads of the first row block). Swept on the 24-block forward,
+        // ms per step: first slot 0 / 2 / 3 / 4 / 5 / 6 / 7 / 8 / 16 with one load per instruction: +0.43 / +0.2 / +0.03 / 0 / -0.05 /
+        // -0.1 / +0.18 / +0.15 / +0.56; from slot 6 every second / third instruction: -0.14 / -0.1.
+        constexpr int LOAD_FIRST = 6, LOAD_EVERY = 2;
         static_assert(HEAD >= TAIL && TAIL >= 1, "every tail fragment is fetched behind a head row block");
         bf16x8_t a[HEAD], at[2][TAIL], b[2][NJ];
         auto a_addr = [&](const char* st, int s, int i) { return reinterpret_cast<const bf16x8_t*>(st + a_off + i * 16 * 128 + (((4 * s + lg) ^ sw) * 16)); };
@@ -253,6 +258,7 @@ __device__ __forceinline__ void gemm_tile(const Prob& pr, const int wg, char* sm
         auto step = [&](int buf, const char* nst, int ns, auto fetch_tag, auto loads_tag) {
             constexpr bool FETCH = decltype(fetch_tag)::value, LOADS = decltype(loads_tag)::value;
             constexpr int NLOADS = LA + LB;
+            static_assert(LOAD_FIRST + NLOADS * LOAD_EVERY <= MI * NJ, "the direct loads fit between the matrix instructions of one step");
             if (FETCH) load_b(nst, ns, buf ^ 1);
 #pragma unroll
             for (int i = 0; i < MI; i++) {
@@ -261,7 +267,7 @@ __device__ __forceinline__ void gemm_tile(const Prob& pr, const int wg, char* sm
                     acc16[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(i < HEAD ? a[i] : at[buf][i - HEAD], b[buf][j], acc16[i][j], 0, 0, 0);
                     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
                     if (FETCH && i == 0) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                       // B fragment j of the next step
-                    if (LOADS && i * NJ + j >= NJ && i * NJ + j < NJ + NLOADS) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // one direct load
+                    if (LOADS && i * NJ + j >= LOAD_FIRST && i * NJ + j < LOAD_FIRST + NLOADS * LOAD_EVERY && (i * NJ + j - LOAD_FIRST) % LOAD_EVERY == 0) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // one direct load
                 }
                 if (FETCH && i < HEAD) {
                     a[i] = *a_addr(nst, ns, i);
