@@ -693,26 +693,32 @@ static int grouped_impl(const GemmBf16Problem* probs, int n, int out_is_f32, int
         if (apart256 < best) { best = apart256; plan = 2; }
         if (apart128 < best) { best = apart128; plan = 3; }
     }
-    // One more plan for a single many-row problem whose 256x256 tiles fill R >= 1 rounds and leave a partial one: its first rows as R
-    // full rounds of 256x256 tiles, its remaining rows together with the few-row problems as 128x128 tiles in a second launch (a
-    // round of those costs 0.62). Only for epilogues that do not look at the row index (a row split would shift the batch boundaries).
-    if (g_gemm_bf16_row_split && nb == 1 && !fp8 && (epi == EPI_BIAS || epi == EPI_BIAS_GELU || epi == EPI_BIAS_SILU || epi == EPI_QKV_NORM)) {
-        const Prob& q = big.p[0];
+    // One more plan when the 256x256 tiles of the many-row problems fill R >= 1 rounds and leave a partial one: everything up to the
+    // last row tile of the last many-row problem that still fits R rounds as 256x256 tiles, the remaining rows of that problem
+    // together with the few-row problems as 128x128 tiles in a second launch (a round of those costs 0.62). Only for epilogues that do
+    // not look at the row index (a row split would shift the batch boundaries).
+    if (g_gemm_bf16_row_split && nb >= 1 && nb + ns <= MAX_PROBS && !fp8 &&
+        (epi == EPI_BIAS || epi == EPI_BIAS_GELU || epi == EPI_BIAS_SILU || epi == EPI_QKV_NORM)) {
+        const Prob& q = big.p[nb - 1];
+        long long before = 0;  // tiles of the many-row problems in front of the one that is split
+        for (int i = 0; i + 1 < nb; i++) before += tiles(big.p[i], 256);
         const int tn = (q.N + 255) / 256, tm = (q.M + 255) / 256;
-        const int R = (int)(big256 / cus), m1 = R > 0 ? (R * cus) / tn : 0;  // row tiles that fit R full rounds
-        if (R > 0 && m1 > 0 && m1 < tm) {
+        const long long R = big256 / cus, avail = R * cus - before;
+        const int m1 = (R > 0 && avail > 0) ? (int)(avail / tn) : 0;  // row tiles of q that fit the R full rounds
+        if (m1 > 0 && m1 < tm) {
             Prob head = q, tail = q;
             head.M = m1 * 256;
             tail.M = q.M - head.M;
             tail.A = q.A + (long long)head.M * q.K;
             tail.out = (char*)q.out + (long long)head.M * q.ldc * (out_is_f32 ? 4 : 2);
-            const double split = rounds(tiles(head, 256), cus) + ROUND128 * rounds(tiles(tail, 128) + small128, 2 * cus);
+            const double split = rounds(before + tiles(head, 256), cus) + ROUND128 * rounds(tiles(tail, 128) + small128, 2 * cus);
             if (split < best) {
                 ProbSet first{}, second{};
-                first.p[0] = head;
+                for (int i = 0; i + 1 < nb; i++) first.p[i] = big.p[i];
+                first.p[nb - 1] = head;
                 second.p[0] = tail;
                 for (int i = 0; i < ns; i++) second.p[1 + i] = small.p[i];
-                SD3_TRY(launch(first, 1, 4));
+                SD3_TRY(launch(first, nb, 4));
                 return launch(second, 1 + ns, 0);
             }
         }

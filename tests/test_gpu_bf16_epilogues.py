@@ -228,6 +228,46 @@ def test_row_split_over_two_launches_gives_identical_bits(epi):
     assert rel_l2(host(base[0][rows]), host(ref)) <= 4e-3
 
 
+def test_row_split_with_two_many_row_problems_gives_identical_bits():
+    """The fused q|k|v launch of a dual-attention block at batch 1: two problems of 4096 rows and one of 154 (2 x 288 + 18 tiles of
+    256x256 on 256 compute units: two full rounds and a partial one). The split leaves the first problem whole, cuts the second behind
+    its last row tile that fits the two rounds and sends the rest with the few-row problem through 128x128 tiles: same bits as the
+    unsplit launch and as either tile shape alone, and a float64 check of rows on both sides of the cut."""
+    g = torch.Generator(device="cuda").manual_seed(77)
+    K, N, Ms = 128, 4608, (4096, 4096, 154)
+    As = [torch.randn((m, K), device="cuda", generator=g).bfloat16() for m in Ms]
+    Wp = [(0.1 * torch.randn((N, K), device="cuda", generator=g)).bfloat16() for _ in Ms]
+    bias = [0.1 * torch.randn(N, device="cuda", generator=g) for _ in Ms]
+    rq, rk = (1 + 0.1 * torch.randn(64, device="cuda", generator=g) for _ in range(2))
+
+    def run(tile, split):
+        outs = [torch.zeros((m, N), device="cuda", dtype=torch.bfloat16) for m in Ms]
+        ps = []
+        for a, w, b, o in zip(As, Wp, bias, outs):
+            p = L.GemmBf16Problem(A=a.data_ptr(), wpacked=w.data_ptr(), bias=b.data_ptr(), out=o.data_ptr(), M=a.shape[0], N=N, K=K)
+            p.rms_q, p.rms_k = rq.data_ptr(), rk.data_ptr()
+            ps.append(p)
+        try:
+            L.call("sd3_tune", b"gemm_bf16_tile", tile)
+            L.call("sd3_tune", b"gemm_bf16_row_split", split)
+            launch(ps, 5, False)
+        finally:
+            L.call("sd3_tune", b"gemm_bf16_tile", 0)
+            L.call("sd3_tune", b"gemm_bf16_row_split", 1)
+        return outs
+
+    base = run(0, 1)
+    for tile, split in ((0, 0), (256, 1), (128, 1)):
+        other = run(tile, split)
+        assert all(torch.equal(a, b) for a, b in zip(other, base)), (tile, split)
+    rows = torch.tensor([0, 3071, 3072, 3073, 4095], device="cuda")  # (512 - 288) // 18 = 12 row tiles of the second problem stay: the cut is at row 3072
+    ref = As[1][rows].double() @ Wp[1].double().t() + bias[1].double()
+    q, k, v = ref.view(len(rows), 3, N // 192, 64).unbind(1)
+    nrm = lambda t, w: t * torch.rsqrt(t.pow(2).mean(-1, keepdim=True) + 1e-6) * w.double()  # noqa: E731
+    ref = torch.stack([nrm(q, rq), nrm(k, rk), v], 1).reshape(len(rows), N)
+    assert rel_l2(host(base[1][rows]), host(ref)) <= 4e-3
+
+
 def test_grouped_gemm_argument_errors():
     none = C.c_void_p(0)
     p = L.GemmBf16Problem(M=4, N=192, K=64)
